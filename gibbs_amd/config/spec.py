@@ -84,12 +84,14 @@ class LayerSpec:
     `mixer`, `ffn_norm`, `ffn`, which may be given in that order as positional arguments; another
     arrangement names whatever roles it wants through `parts` (one norm and two bodies, a block
     without a feed-forward, two mixers, norms after the bodies), and any number of them may be
-    mixers with caches or state of their own."""
+    mixers with caches or state of their own.  `params`: constants of the arrangement itself (a multiplier on
+    what a sublayer adds, for instance)."""
     PRE_NORM_ROLES = ("mixer_norm", "mixer", "ffn_norm", "ffn")
 
     def __init__(self, name: str, arrangement: str, mixer_norm: Optional[NormSpec] = None, mixer: Optional[MixerSpec] = None,
                  ffn_norm: Optional[NormSpec] = None, ffn: Optional[FeedForwardSpec] = None,
-                 parts: Optional[Sequence[Tuple[str, PartSpec]]] = None):
+                 parts: Optional[Sequence[Tuple[str, PartSpec]]] = None, params: Optional[Mapping[str, Any]] = None):
+        self.params: Mapping[str, Any] = dict(params or {})
         self.name = name                    # checkpoint prefix, e.g. "model.layers.3"
         self.arrangement = arrangement
         if parts is None:
@@ -114,7 +116,8 @@ class LayerSpec:
     ffn = property(lambda self: self.part("ffn"))
 
     def __eq__(self, other) -> bool:
-        return isinstance(other, LayerSpec) and (self.name, self.arrangement, self.parts) == (other.name, other.arrangement, other.parts)
+        return (isinstance(other, LayerSpec) and (self.name, self.arrangement, self.parts, self.params)
+                == (other.name, other.arrangement, other.parts, other.params))
 
     def __repr__(self) -> str:
         return f"LayerSpec({self.name!r}, {self.arrangement!r}, parts={self.parts!r})"

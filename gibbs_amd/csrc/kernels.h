@@ -60,6 +60,21 @@ int gibbs_gemm_heads_gated(const void* X, long ldx, long head_x, const void* W, 
 int gibbs_qk_unit_kv(void* rows, long ld, void* kpages, void* vpages, int dtype, const int* pos, const int* row_req,
                      const int* table, int max_pages, int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, int vd,
                      float eps, int unit, int norm_dim, float temp_coef, int temp_every, hipStream_t stream);
+int gibbs_qkv_prepare(void* rows, long ld, void* kpages, void* vpages, int dtype, const float* bias, const float* inv_freq,
+                      int rot, int variant, const float* cs_table, int table_len, void* keep, int keep_mode, int vt,
+                      const float* lambda, const int* pos, const int* row_req, const int* table, int max_pages, int page_size,
+                      int num_pages, int n_rows, int nh, int nkv, int hd, int vd, hipStream_t stream);
+// ---- moe.hip: mixture of experts
+long gibbs_moe_capacity(int n_pairs, int E, int bm);
+int gibbs_moe_tile(int n_pairs, int E);
+int gibbs_moe_route(const void* h, long ldh, int dtype, const float* router, const float* router_bias, const float* shared_gate,
+                    int* chosen, float* weight, float* sgate, int n, int W, int E, int top, hipStream_t stream);
+int gibbs_moe_group(const int* chosen, int n_pairs, int E, int bm, int* sorted_pair, int* pair_pos, int* tile_expert, long cap,
+                    hipStream_t stream);
+int gibbs_moe_gemm(const void* X, long ldx, int top, const int* sorted_pair, const int* tile_expert, long cap, int bm,
+                   const void* w_a, const void* w_b, void* Y, long ldy, int dtype, int O, int I, int act, hipStream_t stream);
+int gibbs_moe_combine(const void* y, const int* pair_pos, const float* weight, const void* shared, const float* sgate, void* out,
+                      int dtype, int n, int top, int W, hipStream_t stream);
 int gibbs_causal_conv_silu(const void* in, long ld, int dtype, const float* taps, float* state, long slot_stride,
                            const int* row_req, const int* cu, const int* slot, float* out, int n_rows, int n_req, int C, int K,
                            int update_state, int single_rows, hipStream_t stream);

@@ -220,6 +220,9 @@ struct Exec {
   bool few_rows;              // a bfloat16 step of so few rows that the weight-streaming products with fused epilogues take it
   bool fused_step;            // and every row is one token of a request of its own (decoded tokens)
   int fused_halves = 0;
+  // rows that a body of this step has published for later bodies (an attention's values, for layers that mix them
+  // into their own), by key; given back when the step ends
+  std::map<int, void*> published;
   Exec(const Plan& plan, const GibbsStepArgs& args);
   void* take(long bytes) {
     void* ptr = arena.take(bytes);
@@ -581,9 +584,18 @@ struct AttnBody : Body {
   const float* bias = nullptr;        // [bias_len, nh]
   const float* bias_t = nullptr;      // the same as [nh, bias_len] divided by the scale: what the matrix-core kernels add to raw scores
   int bias_len = 0;
-  bool extras() const { return vd != hd || unit_qk || temp_every > 0 || bias; }
+  // what gibbs_plan_attention_projection sets: a bias on the projected rows, a sink in the softmax, values that are
+  // published for later layers or mixed with what an earlier layer published (values of their own size with a rotation
+  // on q and k come this way too: `general_prep`)
+  const float* proj_bias = nullptr;   // [qkv.O] float32
+  const float* sink = nullptr;        // [nh]
+  int keep_mode = 0, keep_key = -1, vt = 0;
+  const float* lambda = nullptr;
+  bool general_prep = false;
+  bool extras() const { return !general_prep && (vd != hd || unit_qk || temp_every > 0 || bias); }
   int cache_group() const override { return group; }
-  bool fast() const { return !slopes && !hook && !extras(); }   // the fast kernels know rotations only (or no encoding at all)
+  // the fast kernels know rotations only (or no encoding at all)
+  bool fast() const { return !slopes && !hook && !extras() && !general_prep; }
   // what the kernel that takes the raw projection (q/k norm, rotation, cache write and attention in one) needs
   bool raw_ok() const { return fast() && owns && hd % 16 == 0 && hd <= 256 && (!inv_freq || rot % 16 == 0); }
   bool fusable(bool single) const override { return single && raw_ok() && qkv.I % 8 == 0 && (nh * hd) % 8 == 0; }
@@ -612,13 +624,34 @@ struct AttnBody : Body {
     e.give(att);
   }
   PagedAttention paged() const {
-    return PagedAttention{kpages, vpages, num_pages, page_size, group, nh, nkv, hd, vd, scale, window, slopes, bias, bias_t, bias_len, nullptr};
+    return PagedAttention{kpages, vpages, num_pages, page_size, group, nh, nkv, hd, vd, scale, window, slopes, bias, bias_t, bias_len, sink};
   }
   // q/k norm, rotation and the cache write of the step's rows (a mixer that reads another's cache writes nothing)
   void prepare_rows(Exec& e, void* raw, long ldq) const {
     const int N = e.a.n_rows, kv = owns ? nkv : 0;
     const int* table = e.table(group);
     const int width = e.width(group);
+    if (general_prep) {
+      // bias, rotation, value mixing and the cache write in one pass; the values that later layers mix into theirs
+      // stay in a buffer of the step
+      void* keep = nullptr;
+      if (keep_mode == 1) {
+        keep = e.take((long)N * nkv * vt * e.esize);
+        e.give(e.published[keep_key]);
+        e.published[keep_key] = keep;
+      } else if (keep_mode == 2) {
+        auto it = e.published.find(keep_key);
+        if (it == e.published.end() || !it->second) {
+          if (!e.status) e.status = gibbs_fail("step: an attention mixes in the values of an earlier layer, and none has published them in this step");
+          return;
+        }
+        keep = it->second;
+      }
+      RUN(e, gibbs_qkv_prepare(raw, ldq, owns ? kpages : nullptr, owns ? vpages : nullptr, e.p.dtype, proj_bias, inv_freq, rot, variant, cos_sin,
+                               table_len, keep, keep_mode, vt, lambda, e.a.pos, e.a.row_req, table, width, page_size, num_pages, N, nh, nkv, hd, vd,
+                               e.a.stream));
+      return;
+    }
     if (extras()) {
       RUN(e, gibbs_qk_unit_kv(raw, ldq, owns ? kpages : nullptr, owns ? vpages : nullptr, e.p.dtype, e.a.pos, e.a.row_req, table, width,
                               page_size, num_pages, N, nh, kv, hd, vd, qk_eps, unit_qk, norm_dim, temp_coef, temp_every, e.a.stream));
@@ -889,6 +922,61 @@ struct MlpBody : Body {
   }
 };
 
+// ---- mixture of experts
+// A router picks `top` of E gated feed-forwards for every row (logits and weights in float32, the weights a softmax over the
+// chosen logits alone); the row's result is the weighted sum of theirs, plus a shared expert's times sigmoid(w_sg . h) where
+// the layer has one.  The rows' (row, choice) pairs are sorted by expert on the device and the experts' products run over
+// tiles of pairs that belong to one expert each (moe.hip); the host sees no count, so a step is still one queue of kernels.
+struct MoeBody : Body {
+  const float* router = nullptr;        // [E, hidden] float32
+  const float* router_bias = nullptr;   // [E] or null
+  const void* gate = nullptr;           // [E, F, hidden]
+  const void* up = nullptr;             // [E, F, hidden]
+  const void* down = nullptr;           // [E, hidden, F]
+  int E = 0, top = 0, F = 0, act = 0;
+  Matrix shared_gate_up, shared_down;   // the shared expert (w null: none): [2 SF, hidden], [hidden, SF]
+  int SF = 0, shared_act = 0;
+  const float* shared_gate = nullptr;   // [hidden] float32, or null: the shared expert is added as it is
+  Pending general(Exec& e, void* h) const override {
+    const int N = e.a.n_rows, W = e.p.hidden, pairs = N * top;
+    const int bm = gibbs_moe_tile(pairs, E);
+    const long cap = gibbs_moe_capacity(pairs, E, bm);
+    int* chosen = (int*)e.take((long)pairs * 4);
+    float* weight = (float*)e.take((long)pairs * 4);
+    float* sgate = shared_gate ? (float*)e.take((long)N * 4) : nullptr;
+    RUN(e, gibbs_moe_route(h, W, e.p.dtype, router, router_bias, shared_gate, chosen, weight, sgate, N, W, E, top, e.a.stream));
+    int* sorted = (int*)e.take(cap * 4);
+    int* place = (int*)e.take((long)pairs * 4);
+    int* tile_expert = (int*)e.take(cap / bm * 4);
+    RUN(e, gibbs_moe_group(chosen, pairs, E, bm, sorted, place, tile_expert, cap, e.a.stream));
+    e.give(chosen);
+    void* mid = e.take(cap * F * e.esize);
+    RUN(e, gibbs_moe_gemm(h, W, top, sorted, tile_expert, cap, bm, gate, up, mid, F, e.p.dtype, F, W, act, e.a.stream));
+    void* y = e.take(cap * W * e.esize);
+    RUN(e, gibbs_moe_gemm(mid, F, 0, sorted, tile_expert, cap, bm, down, nullptr, y, W, e.p.dtype, W, F, 0, e.a.stream));
+    e.give(mid);
+    e.give(sorted);
+    e.give(tile_expert);
+    void* shared = nullptr;
+    if (shared_gate_up.w) {
+      void* gu = e.linear(h, shared_gate_up, N, false, false, false, nullptr);
+      void* sy = e.take((long)N * SF * e.esize);
+      RUN(e, gibbs_glu(gu, sy, e.p.dtype, N, SF, shared_act, e.a.stream));
+      e.give(gu);
+      shared = e.linear(sy, shared_down, N, false, false, false, nullptr);
+      e.give(sy);
+    }
+    Pending delta{e.take((long)N * W * e.esize), 1};
+    RUN(e, gibbs_moe_combine(y, place, weight, shared, sgate, delta.data, e.p.dtype, N, top, W, e.a.stream));
+    e.give(shared);
+    e.give(y);
+    e.give(place);
+    e.give(weight);
+    e.give(sgate);
+    return delta;
+  }
+};
+
 // ---- a body from elsewhere
 struct HostBody : Body {
   GibbsHostBody fn = nullptr;
@@ -1032,6 +1120,8 @@ void Exec::run() {
   for (void* r : rows) give(r);
   for (Pending& d : deltas) give(d.data);
   give(mirror);      // (buffers of the caller's are not the arena's: giving them back does nothing)
+  for (auto& kv : published) give(kv.second);
+  published.clear();
   give(embedded);
   give(x);
 }
@@ -1266,6 +1356,45 @@ GIBBS_EXPORT int gibbs_plan_attention_extras(void* plan, int body, int vd, int u
   t->qkv.O = (t->nh + t->nkv) * t->hd + t->nkv * vd;
   t->out.I = t->nh * vd;
   return 0;
+}
+
+GIBBS_EXPORT int gibbs_plan_attention_projection(void* plan, int body, int vd, const float* bias, const float* sink, int keep_mode,
+                                                 int keep_key, int vt, const float* lambda) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  AttnBody* t = p->has_body(body) ? dynamic_cast<AttnBody*>(p->bodies[body].get()) : nullptr;
+  if (!t || vd <= 0 || keep_mode < 0 || keep_mode > 2) { gibbs_fail("plan: body %d is no attention, or bad projection options", body); return -1; }
+  if (t->q_gain || t->k_gain || t->hook || t->unit_qk || t->temp_every > 0 || !t->owns) {
+    gibbs_fail("plan: an attention with projection biases, a sink or value mixing has no q/k norm, no hook and no temperature, and owns its pages");
+    return -1;
+  }
+  if (keep_mode && !(vt > 0 && vt <= vd && keep_key >= 0 && (keep_mode == 1 || lambda))) { gibbs_fail("plan: value mixing needs a key, the values' size and its weight"); return -1; }
+  t->general_prep = true;
+  t->vd = vd; t->proj_bias = bias; t->sink = sink; t->keep_mode = keep_mode; t->keep_key = keep_key; t->vt = vt; t->lambda = lambda;
+  t->qkv.O = (t->nh + t->nkv) * t->hd + t->nkv * vd;
+  t->out.I = t->nh * vd;
+  return 0;
+}
+
+GIBBS_EXPORT int gibbs_plan_body_moe(void* plan, const GibbsMoeSpec* d) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  if (!d || !(d->router && d->gate && d->up && d->down && d->experts > 0 && d->experts <= 1024 && d->top > 0 && d->top <= d->experts && d->F > 0 &&
+              d->act >= 0 && d->act < 4 && (!d->shared_gate_up || (d->shared_down && d->shared_F > 0 && d->shared_act >= 0 && d->shared_act < 4)) &&
+              (!d->shared_gate || d->shared_gate_up))) {
+    gibbs_fail("plan: bad mixture of experts");
+    return -1;
+  }
+  auto b = std::make_unique<MoeBody>();
+  b->router = d->router; b->router_bias = d->router_bias; b->gate = d->gate; b->up = d->up; b->down = d->down;
+  b->E = d->experts; b->top = d->top; b->F = d->F; b->act = d->act;
+  if (d->shared_gate_up) {
+    b->shared_gate_up = Matrix{d->shared_gate_up, nullptr, 2 * d->shared_F, p->hidden};
+    b->shared_down = Matrix{d->shared_down, nullptr, p->hidden, d->shared_F};
+    b->SF = d->shared_F; b->shared_act = d->shared_act; b->shared_gate = d->shared_gate;
+  }
+  p->bodies.push_back(std::move(b));
+  return (int)p->bodies.size() - 1;
 }
 
 GIBBS_EXPORT int gibbs_plan_glu_clamped(void* plan, int body, float alpha, float limit) {

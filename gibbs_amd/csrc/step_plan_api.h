@@ -82,6 +82,25 @@ int gibbs_plan_embedding(void* plan, float scale, const float* inv_freq);
 // Projected rows are then [q: nh*hd | k: nkv*hd | v: nkv*vd].
 int gibbs_plan_attention_extras(void* plan, int body, int vd, int unit_qk, int norm_dim, float temp_coef, int temp_every,
                                 const float* bias, const float* bias_t, int bias_len);
+// An attention body with a rotation (or none) may have: values of head size vd; bias [qkv rows] (float32) added to the
+// projected rows; sink [heads]: a term exp(sink[h]) in the softmax's denominator without key or value; value mixing:
+// keep_mode 1 publishes the step's values (the first vt channels of every value head) under keep_key for later layers,
+// keep_mode 2 mixes what was published under keep_key into its own, v <- (1 - *lambda) v + *lambda v_published, before they
+// are cached.  Projected rows are then [q: nh*hd | k: nkv*hd | v: nkv*vd].
+int gibbs_plan_attention_projection(void* plan, int body, int vd, const float* bias, const float* sink, int keep_mode,
+                                    int keep_key, int vt, const float* lambda);
+// Mixture of experts: router [experts, hidden] and router_bias [experts] (float32); gate, up [experts, F, hidden] and down
+// [experts, hidden, F]; every row takes its `top` experts with the largest logits, weighted by the softmax over those
+// logits; expert: down(act(gate h) * (up h)).  A shared expert (shared_gate_up [2 shared_F, hidden], shared_down [hidden,
+// shared_F]; null: none) runs for every row and is added, times sigmoid(shared_gate . h) (shared_gate [hidden] float32;
+// null: times 1).
+struct GibbsMoeSpec {
+  const float* router; const float* router_bias;
+  const void* gate; const void* up; const void* down;
+  const void* shared_gate_up; const void* shared_down; const float* shared_gate;
+  int experts, top, F, act, shared_F, shared_act;
+};
+int gibbs_plan_body_moe(void* plan, const struct GibbsMoeSpec* spec);
 // A gated feed-forward body computes min(gate, limit) * sigmoid(alpha * .) * (clamp(up, -limit, limit) + 1) instead.
 int gibbs_plan_glu_clamped(void* plan, int body, float alpha, float limit);
 

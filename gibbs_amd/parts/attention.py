@@ -13,6 +13,13 @@ as tables and every fast path stays open; an encoding that changes q and k itsel
 called back between the q/k norm and the cache write, and one that biases the scores by distance
 (`score_slopes`) takes the plain attention kernel, which knows such a bias.  Which kernels a step
 takes is decided where the step runs (csrc/step_plan.hip).
+
+Further options, each a parameter of the spec: `bias` (q, k and v projections have biases: tensors `q_bias`,
+`k_bias`, `v_bias`), `sink` (a learned number per head, tensor `sink`, whose exponential joins the softmax's
+denominator without key or value and without the score's scale), `v_head_dim` (values of a head size of their
+own), and `value_mix` = {"key": k, "publish": bool}: the layer that publishes hands its values of the step's rows
+to the later layers of the same key, which cache and use  v <- (1 - lambda) v + lambda v_published  with their
+own lambda (tensor `value_mix`, one number; the publishing layer declares it too and never reads it).
 """
 from __future__ import annotations
 
@@ -41,6 +48,13 @@ class AttentionMixer(Mixer):
         # (`qk_norm: "unit"`); q times 1 + coef * log(1 + (position + 1) div every) (`q_temperature`)
         self.v_head_dim = int(p.get("v_head_dim") or self.head_dim)
         self.q_temperature = p.get("q_temperature")
+        self.has_bias, self.has_sink = bool(p.get("bias")), bool(p.get("sink"))
+        self.value_mix = p.get("value_mix")
+        if self.value_mix is not None and (self.source is not None or int(self.value_mix["key"]) < 0):
+            raise ValueError("value mixing needs a key >= 0 and a mixer that owns its pages")
+        if (self.has_bias or self.has_sink or self.value_mix is not None) and (self.qk_norm is not None or self.q_temperature is not None
+                                                                              or self.source is not None):
+            raise ValueError("projection biases, a sink and value mixing go with neither a q/k norm nor a temperature nor another layer's cache")
         if self.heads % self.kv_heads:
             raise ValueError(f"{self.heads} heads are not a multiple of {self.kv_heads} kv heads")
         if self.qk_norm not in (None, "before", "unit"):
@@ -92,9 +106,23 @@ class AttentionMixer(Mixer):
             decls.append(TensorDecl(t["q_norm"], (hd,), FLOAT32, init="gain"))
             if self.source is None:
                 decls.append(TensorDecl(t["k_norm"], (hd,), FLOAT32, init="gain"))
+        if self.has_bias:
+            decls += [TensorDecl(t["q_bias"], (self.heads * hd,), FLOAT32, init="bias"),
+                      TensorDecl(t["k_bias"], (self.kv_heads * hd,), FLOAT32, init="bias"),
+                      TensorDecl(t["v_bias"], (self.kv_heads * vd,), FLOAT32, init="bias")]
+        if self.has_sink:
+            decls.append(TensorDecl(t["sink"], (self.heads,), FLOAT32, init="bias"))
+        if self.value_mix is not None:
+            decls.append(TensorDecl(t["value_mix"], (), FLOAT32, init="bias"))
         if self.position is not None:
             decls += self.position.tensor_decls()
         return decls
+
+    def projection_options(self) -> bool:
+        """Options that take the preparation of the step's rows with biases, partial rotation and value mixing."""
+        rotated_own_values = (self.v_head_dim != self.head_dim and self.qk_norm is None and self.q_temperature is None
+                              and self.spec.position is not None and self.spec.position.kind == "rope")
+        return self.has_bias or self.has_sink or self.value_mix is not None or rotated_own_values
 
     def bind(self, weights: WeightStore, rt: Runtime) -> None:
         self.rt = rt
@@ -106,8 +134,8 @@ class AttentionMixer(Mixer):
         # out-projection: products with them are exactly zero).
         self.padded_dim = None
         pad = -(-max(self.head_dim, self.v_head_dim) // 16) * 16
-        if (rt.act_dtype == torch.bfloat16 and self.source is None and self.qk_norm == "unit" and pad <= 128
-                and (self.head_dim, self.v_head_dim) != (pad, pad)):
+        if (rt.act_dtype == torch.bfloat16 and self.source is None and (self.qk_norm == "unit" or self.projection_options())
+                and pad <= 128 and (self.head_dim, self.v_head_dim) != (pad, pad)):
             self.padded_dim = pad
             wq = self._pad_heads(wq, self.heads, self.head_dim, pad, rows=True)
             w_out = self._pad_heads(w_out, self.heads, self.v_head_dim, pad, rows=False)
@@ -122,6 +150,21 @@ class AttentionMixer(Mixer):
             self.w_qkv = wq
         self.w_out = w_out.contiguous()
         self.p_qkv = self.p_out = None
+        # biases in the layout of a projected row (heads as they are stored), the sink and the mixing weight
+        self.proj_bias = self.sinks = self.mix_weight = None
+        if self.has_bias:
+            def stored(b, heads, dim, size):
+                out = torch.zeros((heads, size), dtype=torch.float32, device=b.device)
+                out[:, :dim] = b.view(heads, dim)
+                return out.view(-1)
+            hd_s, vd_s = self.stored_dims()
+            self.proj_bias = torch.cat([stored(weights[t["q_bias"]], self.heads, self.head_dim, hd_s),
+                                        stored(weights[t["k_bias"]], self.kv_heads, self.head_dim, hd_s),
+                                        stored(weights[t["v_bias"]], self.kv_heads, self.v_head_dim, vd_s)]).contiguous()
+        if self.has_sink:
+            self.sinks = weights[t["sink"]].contiguous()
+        if self.value_mix is not None and not self.value_mix.get("publish"):
+            self.mix_weight = weights[t["value_mix"]].reshape(1).contiguous()
         self.q_gain = weights[t["q_norm"]] if self.qk_norm == "before" else None
         self.k_gain = weights[t["k_norm"]] if self.qk_norm == "before" and self.source is None else None
         self.rot, self.slopes, self.pos_hook, self.score_bias = None, None, False, None
@@ -146,7 +189,7 @@ class AttentionMixer(Mixer):
         return [(self.heads * self.head_dim + kv, self.hidden), (self.hidden, self.heads * self.v_head_dim)]
 
     def small_tensors(self):
-        own = [t for t in (self.q_gain, self.k_gain, self.slopes) if t is not None]   # (a score table is the position's)
+        own = [t for t in (self.q_gain, self.k_gain, self.slopes, self.proj_bias, self.sinks, self.mix_weight) if t is not None]   # (a score table is the position's)
         return own + ([] if self.position is None else list(self.position.small_tensors()))
 
     def fold_input_gain(self, gain: torch.Tensor) -> None:
@@ -159,8 +202,8 @@ class AttentionMixer(Mixer):
 
     def extras(self) -> bool:
         """Options that take the general preparation of the step's rows (no rotation, no gains)."""
-        return (self.v_head_dim != self.head_dim or self.qk_norm == "unit" or self.q_temperature is not None
-                or self.score_bias is not None)
+        return not self.projection_options() and (self.v_head_dim != self.head_dim or self.qk_norm == "unit"
+                                                  or self.q_temperature is not None or self.score_bias is not None)
 
     def emit(self, plan, cache) -> int:
         hd, vd = self.stored_dims()
@@ -173,6 +216,13 @@ class AttentionMixer(Mixer):
             plan.attention_extras(body, v_head_dim=vd, unit_qk=self.qk_norm == "unit", temp_coef=float(temp["coef"]),
                                   temp_every=int(temp["every"]), bias=self.score_bias, bias_over_scale=self.score_bias_over_scale,
                                   norm_dim=self.head_dim)
+        if self.projection_options():
+            if hook is not None or self.slopes is not None or self.score_bias is not None:
+                raise ValueError("projection biases, a sink and value mixing go with a rotation or no position encoding")
+            mix = self.value_mix
+            plan.attention_projection(body, v_head_dim=vd, bias=self.proj_bias, sink=self.sinks,
+                                      keep_mode=0 if mix is None else (1 if mix.get("publish") else 2),
+                                      keep_key=-1 if mix is None else int(mix["key"]), value_dim=self.v_head_dim, weight=self.mix_weight)
         return body
 
     def _emit_body(self, plan, cache, hook, head_dim: int) -> int:

@@ -101,6 +101,43 @@ class ParallelNormsBlock(Block):
             plan.add(delta)
 
 
+@register_arrangement("sandwich")
+class SandwichBlock(Block):
+    """Sublayers with a norm on both sides, the normed result times a constant:
+
+        x = x + mult * norm1b(mixer(norm1(x)));   x = x + mult * norm2b(ffn(norm2(x)))
+
+    Roles: `norm1`, `mixer`, `norm1b`, and optionally `norm2`, `ffn`, `norm2b` (a layer without a feed-forward).
+    `mult` is the layer spec's `params["residual_mult"]` (default 1); it is multiplied into the gains of the norms
+    behind the sublayers when the weights are bound.  The norm of a sublayer's result and its addition into the
+    float32 stream are one pass (`plan.add_normed`)."""
+
+    def __init__(self, spec, hidden, layer_index):
+        super().__init__(spec, hidden, layer_index)
+        self.has_ffn = "ffn" in self.named
+        self.mult = float(spec.params.get("residual_mult", 1.0))
+        want = ["norm1", "mixer", "norm1b"] + (["norm2", "norm2b"] if self.has_ffn else [])
+        missing = [r for r in want if r not in self.named]
+        if missing:
+            raise ValueError(f"layer {spec.name!r} lacks the parts {missing}")
+
+    def bind(self, weights, rt: Runtime) -> None:
+        super().bind(weights, rt)
+        if self.mult != 1.0:
+            for norm in [self.norm1b] + ([self.norm2b] if self.has_ffn else []):
+                norm.gain = (norm.gain * self.mult).contiguous()
+
+    def emit(self, plan, caches) -> None:
+        subs = [(self.norm1, lambda: self.mixer.emit(plan, caches["mixer"]), self.norm1b)]
+        if self.has_ffn:
+            subs.append((self.norm2, lambda: self.ffn.emit(plan), self.norm2b))
+        for before, body, after in subs:
+            h = plan.normed(before.emit(plan))
+            delta = plan.apply(body(), h)
+            plan.drop(h)
+            plan.add_normed(after.emit(plan), delta)
+
+
 @register_connection("hyper")
 class HyperConnection(Connection):
     """A sublayer over S residual streams x_1 .. x_S: it reads u = sum_s in[s] x_s and, with its result y, writes all

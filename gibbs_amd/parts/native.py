@@ -61,6 +61,13 @@ class LatentSpec(ctypes.Structure):
                 ("num_pages", c_int), ("page_size", c_int), ("group", c_int), ("scale", ctypes.c_float), ("eps", ctypes.c_float)]
 
 
+class MoeSpec(ctypes.Structure):
+    """GibbsMoeSpec of csrc/step_plan_api.h."""
+    _fields_ = [("router", c_void_p), ("router_bias", c_void_p), ("gate", c_void_p), ("up", c_void_p), ("down", c_void_p),
+                ("shared_gate_up", c_void_p), ("shared_down", c_void_p), ("shared_gate", c_void_p),
+                ("experts", c_int), ("top", c_int), ("F", c_int), ("act", c_int), ("shared_F", c_int), ("shared_act", c_int)]
+
+
 HOST_BODY = CFUNCTYPE(c_int, c_void_p, POINTER(StepArgs), c_void_p, c_void_p)
 HOST_NORM = CFUNCTYPE(c_int, c_void_p, POINTER(StepArgs), c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p)
 HOST_ROWS = CFUNCTYPE(c_int, c_void_p, POINTER(StepArgs), c_void_p, c_long)
@@ -86,6 +93,8 @@ def declare(lib) -> None:
         "gibbs_plan_embedding": ([P, F, P], I),
         "gibbs_plan_attention_extras": ([P, I, I, I, I, F, I, P, P, I], I),
         "gibbs_plan_glu_clamped": ([P, I, F, F], I),
+        "gibbs_plan_attention_projection": ([P, I, I, P, P, I, I, I, P], I),
+        "gibbs_plan_body_moe": ([P, POINTER(MoeSpec)], I),
         "gibbs_plan_body_delta": ([P, POINTER(DeltaSpec)], I),
         "gibbs_plan_body_time_mix": ([P, POINTER(TimeMixSpec)], I),
         "gibbs_plan_norm_layer": ([P, P, P, F], I),
@@ -259,6 +268,25 @@ class NativePlan:
         self._made(L.library().gibbs_plan_attention_extras(self.handle, int(body), int(v_head_dim), int(unit_qk), int(norm_dim),
                                                            float(temp_coef), int(temp_every), b, bt,
                                                            0 if bias is None else int(bias.shape[0])))
+
+    def attention_projection(self, body: int, *, v_head_dim: int, bias, sink, keep_mode: int, keep_key: int, value_dim: int,
+                             weight) -> None:
+        """Options of an attention body with a rotation (or no encoding): values of a head size of their own, a float32
+        bias on the projected rows, a sink per head in the softmax, and value mixing (`keep_mode` 1: the step's values
+        are published under `keep_key`; 2: what was published is mixed in with `weight`, one float32 on the device)."""
+        b, s, w = self._held(bias, sink, weight)
+        self._made(L.library().gibbs_plan_attention_projection(self.handle, int(body), int(v_head_dim), b, s, int(keep_mode),
+                                                               int(keep_key), int(value_dim), w))
+
+    def moe(self, m) -> int:
+        """The mixture-of-experts feed-forward `m` (parts/moe.py)."""
+        from ..ops import ACTIVATIONS
+        d = MoeSpec()
+        d.router, d.router_bias, d.gate, d.up, d.down = self._held(m.router, m.router_bias, m.w_gate, m.w_up, m.w_down)
+        d.shared_gate_up, d.shared_down, d.shared_gate = self._held(m.shared_gate_up, m.shared_down, m.shared_gate)
+        d.experts, d.top, d.F, d.act = m.experts, m.top, m.inter, ACTIVATIONS[m.activation]
+        d.shared_F, d.shared_act = m.shared_inter, ACTIVATIONS[m.shared_activation]
+        return self._made(L.library().gibbs_plan_body_moe(self.handle, ctypes.byref(d)))
 
     def glu_clamped(self, body: int, *, alpha: float, limit: float) -> None:
         self._made(L.library().gibbs_plan_glu_clamped(self.handle, int(body), float(alpha), float(limit)))

@@ -1,7 +1,7 @@
 """Rotary position encoding: the table of inverse frequencies and the pairing variant that an
 attention mixer hands to its kernel.
 
-inv_freq[j] = 1 / theta^(2j / rotary_dim); with `precision: "f32"` every step of that is a
+inv_freq[j] = 1 / theta^(2j / rotary_dim), divided by `scaling_factor` where positions are scaled linearly; with `precision: "f32"` every step of that is a
 float32 operation, as LFM2's spec asks (src/arch/gen.rs:154-164,
 arch/families/lfm2.json5:64).  The angle of position p is float32(p) * inv_freq[j]
 (src/graph/cpu.rs:673); variant `half_split` turns the pair (j, j + rot/2),
@@ -24,8 +24,13 @@ from .base import PositionEncoding, Rotation, Runtime, register_position
 MAX_TABLE_POSITIONS = 1 << 20   # 8 bytes * rotary_dim / 2 each
 
 
-def rope_inv_freq(rotary_dim: int, theta: float, precision: str = "f64") -> np.ndarray:
+def rope_inv_freq(rotary_dim: int, theta: float, precision: str = "f64", factor: float = 1.0) -> np.ndarray:
+    """`factor`: linear scaling of the positions: every frequency is divided by it (before it is rounded to float32)."""
     half = rotary_dim // 2
+    if factor != 1.0:
+        if precision != "f64":
+            raise ValueError("a scaling factor on the rotation's frequencies is computed in float64")
+        return np.array([1.0 / (float(theta) ** (2.0 * j / rotary_dim)) / float(factor) for j in range(half)]).astype(np.float32)
     if precision == "f32":
         t = np.float32(theta)
         return np.array([np.float32(1.0) / np.power(t, np.float32(2 * j) / np.float32(rotary_dim), dtype=np.float32)
@@ -44,6 +49,9 @@ class RotaryPosition(PositionEncoding):
         self.variant = p.get("variant", "half_split")
         self.theta = float(p["theta"])
         self.precision = p.get("precision", "f64")
+        self.factor = float(p.get("scaling_factor", 1.0))
+        if not self.factor > 0:
+            raise ValueError(f"the rotation's scaling factor {self.factor} must be positive")
         if self.rotary_dim <= 0 or self.rotary_dim % 2 or self.rotary_dim > head_dim:
             raise ValueError(f"rotary_dim {self.rotary_dim} must be even and within the head size {head_dim}")
         if self.variant not in ("half_split", "interleaved"):
@@ -52,9 +60,9 @@ class RotaryPosition(PositionEncoding):
     def bind(self, weights: WeightStore, rt: Runtime) -> None:
         self.rt = rt
         n_pos = min(int(rt.max_positions), MAX_TABLE_POSITIONS)
-        key = ("rope", self.rotary_dim, self.theta, self.precision, n_pos)
+        key = ("rope", self.rotary_dim, self.theta, self.precision, self.factor, n_pos)
         if key not in rt.shared:        # the layers of a model that have the same encoding share one table
-            inv_freq = torch.from_numpy(rope_inv_freq(self.rotary_dim, self.theta, self.precision)).to(rt.device)
+            inv_freq = torch.from_numpy(rope_inv_freq(self.rotary_dim, self.theta, self.precision, self.factor)).to(rt.device)
             rt.shared[key] = (inv_freq, ops.rope_table(inv_freq, n_pos) if n_pos > 0 else None)
         self.inv_freq, self.cos_sin = rt.shared[key]
 
