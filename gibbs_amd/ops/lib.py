@@ -85,6 +85,14 @@ _SIGNATURES = {
                                c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gibbs_qk_unit_kv": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                          c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_float, c_int, c_void_p],
+    "gibbs_qkv_prepare": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_int,
+                          c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "gibbs_moe_route": [c_void_p, c_long, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                        c_void_p],
+    "gibbs_moe_group": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p],
+    "gibbs_moe_gemm": [c_void_p, c_long, c_int, c_void_p, c_void_p, c_long, c_int, c_void_p, c_void_p, c_void_p, c_long, c_int, c_int,
+                       c_int, c_int, c_void_p],
+    "gibbs_moe_combine": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "gibbs_causal_conv_silu": [c_void_p, c_long, c_int, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gibbs_delta_rule": [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p, c_long, c_void_p,
@@ -110,6 +118,8 @@ _SIGNATURES = {
 
 
 _VALUE_SIGNATURES = {
+    "gibbs_moe_capacity": ([c_int, c_int, c_int], c_long),
+    "gibbs_moe_tile": ([c_int, c_int], c_int),
     "gibbs_pair_layout_below_tiles": ([], c_int),
     "gibbs_rule_skinny_splits": ([c_int, c_int, c_int, c_int, c_int], c_int),
     "gibbs_rule_decode_splits": ([c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p], None),

@@ -113,4 +113,4 @@ def write_safetensors(path: str, tensors: Mapping[str, torch.Tensor] | Iterable[
         f.write(blob)
         for _, t in items:
             t = t.detach().contiguous().cpu()
-            f.write(t.view(torch.uint8).numpy().tobytes() if t.numel() else b"")
+            f.write(t.reshape(-1).view(torch.uint8).numpy().tobytes() if t.numel() else b"")
