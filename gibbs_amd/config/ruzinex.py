@@ -78,9 +78,9 @@ class RuzinexConfig(ArchConfig):
                 if factor is not None and not float(factor) > 0:
                     raise ConfigError(f"layer {i}: a scaling factor of {factor}")
             if m.get("v_mix"):
-                size = int(m["kv_heads"]) * int(m["vdim"])
+                size = (int(m["kv_heads"]), int(m["vdim"]))
                 if mixed is not None and mixed != size:
-                    raise ConfigError(f"layer {i}: value mixing needs values of {mixed} numbers a token, this layer has {size}")
+                    raise ConfigError(f"layer {i}: value mixing needs {mixed[0]} value heads of {mixed[1]}, this layer has {size[0]} of {size[1]}")
                 mixed = size
             elif tensors is not None and f"l{i}.mix.vmix" in tensors:
                 unread.append((f"l{i}.mix.vmix", tuple(int(s) for s in tensors[f"l{i}.mix.vmix"])))

@@ -107,10 +107,21 @@ def route(h, router, bias, top: int):
     return chosen, e / e.sum(-1, keepdims=True)
 
 
-def expert_feed_forward(h, w, p: str, mlp: dict):
+def route_margin(h, router, bias, top: int):
+    """How clear every row's choice is: the gap between its last chosen logit and the next one, in units of the row's
+    spread of logits (infinite when every expert is chosen)."""
+    z = np.sort(h @ router.T + bias, axis=-1)[:, ::-1]
+    if top >= z.shape[1]:
+        return np.full(z.shape[0], np.inf)
+    return (z[:, top - 1] - z[:, top]) / (z.std(-1) + 1e-30)
+
+
+def expert_feed_forward(h, w, p: str, mlp: dict, margins_out=None):
     """Weighted sum of each token's chosen experts, plus the shared expert times sigmoid(sg h) where the layer has one."""
     n, top = int(mlp["router"]["experts"]), int(mlp["router"]["top"])
     chosen, weight = route(h, w[p + "router"], w[p + "router.b"], top)
+    if margins_out is not None:
+        margins_out.append(route_margin(h, w[p + "router"], w[p + "router.b"], top))
     out = np.zeros((h.shape[0], w[p + "e0.down"].shape[0]), dtype=F64)
     for e in range(n):
         rows, slot = np.nonzero(chosen == e)
@@ -121,20 +132,21 @@ def expert_feed_forward(h, w, p: str, mlp: dict):
     return out
 
 
-def feed_forward(h, w, p: str, mlp: dict):
+def feed_forward(h, w, p: str, mlp: dict, margins_out=None):
     if mlp["kind"] == "dense":
         return gated(h, w, p, gelu_tanh)
     if mlp["kind"] == "moe":
-        return expert_feed_forward(h, w, p, mlp)
+        return expert_feed_forward(h, w, p, mlp, margins_out)
     raise ValueError(mlp["kind"])
 
 
 # --------------------------------------------------------------------------- the model
-def forward(cfg: dict, w: dict, tokens, layers_out=None) -> np.ndarray:
-    """Logits [T, vocab] of one sequence.  `layers_out`: a list that takes the residual stream after every layer."""
+def forward(cfg: dict, w: dict, tokens, layers_out=None, margins_out=None) -> np.ndarray:
+    """Logits [T, vocab] of one sequence.  `layers_out`: a list that takes the residual stream after every layer;
+    `margins_out`: a list that takes every expert layer's `route_margin` of the tokens."""
     tokens = np.asarray(tokens, dtype=np.int64)
     positions = np.arange(len(tokens))
-    eps, mult = float(cfg["norm"]["eps"]), float(cfg["residual_mult"])
+    eps, mult = float(cfg["norm"]["eps"]), float(cfg.get("residual_mult", 1.0))
     x = w["embed"][tokens].astype(F64)
     v_first = None
     for i, layer in enumerate(cfg["layers"]):
@@ -147,7 +159,7 @@ def forward(cfg: dict, w: dict, tokens, layers_out=None) -> np.ndarray:
             v_first = v
         x = x + mult * rms_norm(d, w[p + "norm1b"], eps)
         if layer.get("mlp") is not None:
-            d = feed_forward(rms_norm(x, w[p + "norm2"], eps), w, p + "mlp.", layer["mlp"])
+            d = feed_forward(rms_norm(x, w[p + "norm2"], eps), w, p + "mlp.", layer["mlp"], margins_out)
             x = x + mult * rms_norm(d, w[p + "norm2b"], eps)
         if layers_out is not None:
             layers_out.append(x.copy())

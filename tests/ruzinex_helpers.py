@@ -45,7 +45,7 @@ RUZINEX_A = {
     "layers": [
         _layer(_mix(6, 3, 20, 12, 0.2, rot=(1000.0, 10, 4.0)), dense(150)),
         _layer(_mix(6, 3, 20, 12, 0.25, rot=(1000.0, 20, None), v_mix=True), moe(5, 2, 30, shared=44)),
-        _layer(_mix(4, 2, 14, 18, 0.3, rot=(300.0, 6, 2.0), v_mix=True), None),
+        _layer(_mix(3, 3, 14, 12, 0.3, rot=(300.0, 6, 2.0), v_mix=True), None),
         _layer(_mix(9, 3, 12, 12, 0.22, rot=(50000.0, 12, 1.5), v_mix=True), moe(3, 3, 50)),
     ],
 }
@@ -56,7 +56,7 @@ RUZINEX_B = {
     "layers": [
         _layer(_mix(8, 2, 64, 64, 0.125, rot=(10000.0, 64, None), v_mix=True), moe(8, 1, 64, shared=64)),
         _layer(_mix(8, 2, 64, 64, 0.125, rot=(10000.0, 64, None), v_mix=True), dense(256)),
-        _layer(_mix(4, 4, 32, 32, 0.18, rot=(10000.0, 16, 8.0), v_mix=True), moe(16, 4, 32)),
+        _layer(_mix(8, 2, 32, 64, 0.18, rot=(10000.0, 16, 8.0), v_mix=True), moe(16, 4, 32)),
     ],
 }
 # C: values larger than keys (in bfloat16 stored at one padded size), no grouping of heads, no value mixing, no
@@ -117,6 +117,7 @@ def load_model_dir(model_dir: str):
 
 _models: dict = {}
 _logits: dict = {}
+_margins: dict = {}
 
 
 def plain_logits(model_dir: str, ids) -> np.ndarray:
@@ -125,5 +126,13 @@ def plain_logits(model_dir: str, ids) -> np.ndarray:
         if model_dir not in _models:
             _models[model_dir] = load_model_dir(model_dir)
         cfg, w = _models[model_dir]
-        _logits[key] = Z.forward(cfg, w, list(ids))
+        margins = []
+        _logits[key] = Z.forward(cfg, w, list(ids), margins_out=margins)
+        _margins[key] = np.min(margins, axis=0) if margins else np.full(len(ids), np.inf)
     return _logits[key]
+
+
+def plain_margins(model_dir: str, ids) -> np.ndarray:
+    """Per token, how clear the least clear choice of experts among the model's layers is (`Z.route_margin`)."""
+    plain_logits(model_dir, ids)
+    return _margins[(model_dir, tuple(ids))]

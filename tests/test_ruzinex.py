@@ -53,7 +53,7 @@ def test_declared_tensors():
     assert "l2.norm2" not in shapes and shapes["l2.norm1b"] == (100,) and shapes["l3.norm2b"] == (100,)
     need = model.cache_needs()
     assert (need[0].kv_heads, need[0].head_dim, need[0].value_dim, need[0].window) == (3, 20, 12, None)
-    assert (need[2].kv_heads, need[2].head_dim, need[2].value_dim) == (2, 14, 18) and all(not s for s in model.state_needs())
+    assert (need[2].kv_heads, need[2].head_dim, need[2].value_dim) == (3, 14, 12) and all(not s for s in model.state_needs())
 
 
 def test_what_the_checkpoint_holds_decides_the_optional_tensors():
@@ -84,6 +84,7 @@ def test_bad_configurations_are_refused():
     broken(lambda c: c["layers"][0]["mixer"]["rot"].update(dims=22))
     broken(lambda c: c["layers"][1]["mlp"]["router"].update(top=6))
     broken(lambda c: c["layers"][3]["mixer"].update(vdim=13))          # its values no longer fit the ones it mixes in
+    broken(lambda c: c["layers"][2]["mixer"].update(heads=4, kv_heads=2, vdim=18))   # as many numbers, in other heads
     broken(lambda c: c["layers"][0]["mlp"].update(kind="sparse"))
     broken(lambda c: c.pop("width"))
 

@@ -22,11 +22,12 @@ DTYPES = ["float32", "bfloat16"]
 NAMES = ["A", "B", "C", "D"]
 LENGTHS = {"A": 150, "B": 330, "C": 120, "D": 90}
 # bfloat16 against the plain implementation, per row: relative L2 error of the logits.  A router's choice between two
-# experts whose logits differ by less than the rounding of its input may fall the other way than in float64, and that
-# row (and what later rows read of it) is then off by more: a few rows in a hundred may exceed the bound, none by much.
+# experts whose logits differ by less than the rounding of its input may fall the other way than in float64: rows whose
+# least clear choice (`route_margin`) is below CLEAR_CHOICE are not held to the bound, and of the others one in a
+# hundred may exceed it (a row that attends to a token whose choice fell the other way).
 BF16_REL_L2 = 0.05
-BF16_ROWS_OVER = 0.03
-BF16_WORST = 0.5
+BF16_ROWS_OVER = 0.01
+CLEAR_CHOICE = 0.03
 
 
 @pytest.fixture(scope="module")
@@ -48,7 +49,7 @@ def make_engine(model_dir, dtype, **kw):
     return Engine(model_dir, dtype=dtype, **kw)
 
 
-def close(got, want, dtype, what):
+def close(got, want, dtype, what, margins=None):
     got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
     assert got.shape == want.shape, (what, got.shape, want.shape)
     if dtype == "float32":
@@ -57,9 +58,13 @@ def close(got, want, dtype, what):
         assert err.max() <= bound, f"{what}: max error {err.max():.3e} at row {int(err.argmax())} above {bound:.3e}; first bad row {int((err > bound).argmax())}"
         return
     rel = np.sqrt(((got - want) ** 2).sum(-1) / (want ** 2).sum(-1))
-    over = rel > BF16_REL_L2
-    assert rel.max() <= BF16_WORST and over.sum() <= max(1, BF16_ROWS_OVER * rel.size), \
-        f"{what}: relative L2 error {rel.max():.3e} at row {int(rel.argmax())}; {int(over.sum())} of {rel.size} rows over; first bad row {int(over.argmax())}"
+    assert np.isfinite(rel).all(), what
+    clear = np.ones(rel.size, dtype=bool) if margins is None else np.asarray(margins) >= CLEAR_CHOICE
+    assert clear.sum() >= 0.5 * rel.size, f"{what}: only {int(clear.sum())} of {rel.size} rows have clear choices of experts"
+    over = (rel > BF16_REL_L2) & clear
+    allowed = 0 if margins is None or np.isinf(margins).all() else max(1, int(BF16_ROWS_OVER * rel.size))
+    assert over.sum() <= allowed, \
+        f"{what}: relative L2 error {rel[clear].max():.3e}; {int(over.sum())} of {int(clear.sum())} rows with clear choices over; first bad row {int(over.argmax())}"
 
 
 def check(model_dir, seqs, got, dtype, what):
@@ -67,7 +72,7 @@ def check(model_dir, seqs, got, dtype, what):
         want = ZH.plain_logits(model_dir, ids)
         places = sorted(p for r, p in got if r == rid)
         assert places, f"{what}: no logits for {rid}"
-        close(np.stack([got[(rid, p)] for p in places]), want[places], dtype, f"{what} request {rid}")
+        close(np.stack([got[(rid, p)] for p in places]), want[places], dtype, f"{what} request {rid}", ZH.plain_margins(model_dir, ids)[places])
 
 
 def vocab_of(model_dir):
