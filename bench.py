@@ -325,7 +325,22 @@ def lfm2_attention_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
     return dict(lfm2_shape(width, ff, layers, vocab), full_attn_idxs=list(range(layers)))
 
 
-BESIDE = {"zokepel": ("Zokepel", zokepel_shape, lfm2_shape), "rukosun": ("Rukosun", rukosun_shape, lfm2_attention_shape)}
+def ruzinex_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
+    """A Ruzinex model of `layers` attention layers whose sizes resemble a real model's at this width: heads of 64 in groups
+    of four with half of every head rotated (positions scaled by 8), values of 64, value mixing in every layer; dense
+    feed-forwards and mixtures of experts in turn, a mixture being 16 experts of an eighth of the dense width of which a
+    token takes 4, beside a shared expert of half the dense width: as many multiplications a token as the dense layer."""
+    heads = width // 64
+    mixer = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 64, "vdim": 64, "scale": 0.125, "v_mix": True,
+             "rot": {"base": 1000000.0, "dims": 32, "scaling": {"factor": 8.0}}}
+    mlps = [{"kind": "dense", "ff": ff},
+            {"kind": "moe", "expert": {"ff": ff // 8}, "router": {"experts": 16, "top": 4}, "shared": {"ff": ff // 2}}]
+    return {"architecture": "Ruzinex", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.7,
+            "layers": [{"type": "attention", "mixer": mixer, "mlp": mlps[i % 2]} for i in range(layers)]}
+
+
+BESIDE = {"zokepel": ("Zokepel", zokepel_shape, lfm2_shape), "rukosun": ("Rukosun", rukosun_shape, lfm2_attention_shape),
+          "ruzinex": ("Ruzinex", ruzinex_shape, lfm2_attention_shape)}
 
 
 def engine_of(shape: dict, dtype: str, max_requests: int, context: int):
@@ -343,7 +358,7 @@ def engine_of(shape: dict, dtype: str, max_requests: int, context: int):
 
 
 def compare_designs(args) -> int:
-    """`--design zokepel` / `--design rukosun`: prefill and decode speed of that design at a few sizes beside LFM2 at equal
+    """`--design zokepel` / `rukosun` / `ruzinex`: prefill and decode speed of that design at a few sizes beside LFM2 at equal
     width, depth, feed-forward and vocabulary (random weights), with the kernels that each one's time goes to.  One
     JSON line."""
     import faulthandler
@@ -405,9 +420,9 @@ def compare_designs(args) -> int:
 
 def main() -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", choices=["lfm2", "zokepel", "rukosun"], default="lfm2",
-                    help="zokepel, rukosun: that design beside LFM2 at equal sizes instead of the headline workload")
-    ap.add_argument("--sizes", choices=["small", "medium", "all"], default="medium", help="sizes of --design zokepel / rukosun")
+    ap.add_argument("--design", choices=["lfm2", "zokepel", "rukosun", "ruzinex"], default="lfm2",
+                    help="zokepel, rukosun, ruzinex: that design beside LFM2 at equal sizes instead of the headline workload")
+    ap.add_argument("--sizes", choices=["small", "medium", "all"], default="medium", help="sizes of --design zokepel / rukosun / ruzinex")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)

@@ -14,8 +14,10 @@
 // A pair's result depends on nothing but its own row and expert (no sum runs over pairs), so where a pair lands
 // among its expert's pairs, which the atomic counters of `group` decide, changes no value: a row's result is the
 // same whatever else is in the batch.  Products: plain FMA in ascending k for float32 and for bfloat16 operands
-// that are not 16-byte aligned; 16 x 16 x 32 matrix-core products for aligned bfloat16 (operands straight from
-// memory: rows of h and of every W are contiguous along k), float32 accumulators, the activation in float32.
+// that are not 16-byte aligned; on the matrix cores for aligned bfloat16, float32 accumulators, the activation in
+// float32: tiles of 16 pairs for steps of few pairs (the experts' matrices are streamed once, a workgroup's four
+// waves split k, operands straight from memory: rows of h and of every W are contiguous along k), tiles of 128
+// pairs beyond (128 x 128 x 64 through LDS, double-buffered, as the framework's tiled product).
 #include "common.h"
 #include "activation.h"
 
@@ -45,40 +47,47 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
     if (lane == 0) sgate[n] = 1.0f / (1.0f + expf(-s));
   }
   __syncthreads();
-  if (threadIdx.x != 0) return;
-  // the `top` largest, in descending order; the lower index among equal logits; then the softmax over them alone
+  if (wave != 0) return;
+  // the `top` largest, in descending order, the lower index among equal logits (one wave: a lane scans its share of
+  // the experts, the lanes' bests are folded by exchanges); a logit that was taken becomes NaN; then the softmax
+  // over the chosen logits alone
   int* mine = chosen + (size_t)n * top;
   float* wts = weight + (size_t)n * top;
-  float best = 0.f;
+  float best = 0.f, sum = 0.f;
   for (int c = 0; c < top; ++c) {
-    int pick = -1;
-    float pv = 0.f;
-    for (int e = 0; e < E; ++e) {
+    float pv = -INFINITY;
+    int pick = 0x7fffffff;
+    for (int e = lane; e < E; e += WAVE) {
       const float v = z[e];
-      if (v != v) continue;
-      bool taken = false;
-      for (int d = 0; d < c; ++d) taken |= mine[d] == e;
-      if (!taken && (pick < 0 || v > pv)) { pick = e; pv = v; }
+      if (v == v && (v > pv || (v == pv && e < pick) || pick == 0x7fffffff)) { pv = v; pick = e; }
     }
-    if (pick < 0) {   // (fewer usable logits than choices: the first expert not taken yet, with no weight)
-      for (int e = 0; e < E && pick < 0; ++e) {
+#pragma unroll
+    for (int o = WAVE / 2; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(pv, o, WAVE);
+      const int op = __shfl_xor(pick, o, WAVE);
+      if (op != 0x7fffffff && (pick == 0x7fffffff || ov > pv || (ov == pv && op < pick))) { pv = ov; pick = op; }
+    }
+    if (pick == 0x7fffffff) {   // (fewer usable logits than choices: the first expert not taken yet, with no weight)
+      for (int e = 0; e < E && pick == 0x7fffffff; ++e) {
         bool taken = false;
         for (int d = 0; d < c; ++d) taken |= mine[d] == e;
         if (!taken) pick = e;
       }
       pv = -INFINITY;
     }
-    mine[c] = pick;
-    wts[c] = pv;
     if (c == 0) best = pv;
+    const float w = pv == -INFINITY ? 0.f : expf(pv - best);
+    sum += w;
+    if (lane == 0) {
+      mine[c] = pick;
+      wts[c] = w;
+      z[pick] = __builtin_nanf("");
+    }
+    __builtin_amdgcn_s_waitcnt(0);   // (the wave's own LDS write above is read by its next scan)
+    __builtin_amdgcn_wave_barrier();
   }
-  float sum = 0.f;
-  for (int c = 0; c < top; ++c) {
-    const float e = wts[c] == -INFINITY ? 0.f : expf(wts[c] - best);
-    wts[c] = e;
-    sum += e;
-  }
-  for (int c = 0; c < top; ++c) wts[c] = sum > 0.f ? wts[c] / sum : 0.f;
+  if (lane == 0)
+    for (int c = 0; c < top; ++c) wts[c] = sum > 0.f ? wts[c] / sum : 0.f;
 }
 
 // ------------------------------------------------------------------------------------------------- group
@@ -187,57 +196,201 @@ __global__ __launch_bounds__(256) void moe_gemm_plain_kernel(const T* __restrict
 }
 
 // ------------------------------------------------------------------------------------------------- products, matrix cores
-// bfloat16, inner size a multiple of 8, rows 16-byte aligned.  W is the first operand (the tile is Y^T = W X^T): lane l
-// holds the 8 values k = (l / 16) * 8 .. + 8 of feature or row l % 16, and its four results are four neighbouring
-// features of row l % 16.  BM 64: a workgroup's four waves take 16 places each and the same 64 features.  BM 16: all
-// four take the same 16 places and 64 features each (256 a workgroup): few pairs, the matrices are streamed once.
+// bfloat16, inner size a multiple of 8, rows 16-byte aligned.
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
-template <int BM, bool GLU>
-__global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16* __restrict__ X, long ldx, int top, const int* __restrict__ sorted_pair,
-                                                            const int* __restrict__ tile_expert, const bf16* __restrict__ Wa,
-                                                            const bf16* __restrict__ Wb, long expert_stride, bf16* __restrict__ Y, long ldy,
-                                                            int O, int I, int act) {
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+
+// Few pairs: a tile is 16 places, a workgroup takes 32 features of it (of both matrices, GLU) and its four waves a
+// quarter of k each, so that the experts' matrices, which are read once, are spread over many workgroups; the waves'
+// sums meet in LDS and the first wave adds them in wave order.  W is the first operand of the 16 x 16 x 32 product (the
+// tile is Y^T = W X^T): lane l holds the 8 values k = (l / 16) * 8 .. + 8 of feature or place l % 16, and its four
+// results are four neighbouring features of place l % 16.  Operands come straight from memory.
+template <bool GLU>
+__global__ __launch_bounds__(256) void moe_gemm_few_kernel(const bf16* __restrict__ X, long ldx, int top, const int* __restrict__ sorted_pair,
+                                                           const int* __restrict__ tile_expert, const bf16* __restrict__ Wa,
+                                                           const bf16* __restrict__ Wb, long expert_stride, bf16* __restrict__ Y, long ldy,
+                                                           int O, int I, int act) {
+  constexpr int NF = 2, NA = GLU ? 2 * NF : NF;    // feature tiles of 16 a workgroup; accumulators a wave
+  __shared__ float part[4][NA][WAVE][4];
   const int tile = blockIdx.y, e = tile_expert[tile];
   if (e < 0) return;
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, lr = lane % 16, lg = lane / 16;
-  const int place = tile * BM + (BM == 64 ? wave * 16 : 0) + lr;
-  const int col0 = BM == 64 ? blockIdx.x * 64 : blockIdx.x * 256 + wave * 64;
-  if (col0 >= O) return;
+  const int place = tile * 16 + lr;
+  const int col0 = blockIdx.x * (16 * NF);
   const int pair = sorted_pair[place];
   const long src = pair < 0 ? -1 : (top > 0 ? pair / top : place);
   const bf16* xr = X + (size_t)(src < 0 ? 0 : src) * ldx;
   const bf16* wa = Wa + (size_t)e * expert_stride;
   const bf16* wb = GLU ? Wb + (size_t)e * expert_stride : nullptr;
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-  floatx4 acc_a[4], acc_b[4];
+  floatx4 acc[NA];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) acc_a[t] = acc_b[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < I; k0 += 32) {
+  for (int t = 0; t < NA; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+  // wave w takes the steps of 32 along k whose number is w modulo 4
+  for (int k0 = wave * 32; k0 < I; k0 += 128) {
     const int k = k0 + lg * 8;
     const bf16x8 x8 = (src >= 0 && k < I) ? *(const bf16x8*)(xr + k) : zero8;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
+    for (int t = 0; t < NF; ++t) {
       const int col = col0 + t * 16 + lr;
       const bool in = col < O && k < I;
       const bf16x8 a8 = in ? *(const bf16x8*)(wa + (size_t)col * I + k) : zero8;
-      acc_a[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a8, x8, acc_a[t], 0, 0, 0);
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a8, x8, acc[t], 0, 0, 0);
       if (GLU) {
         const bf16x8 b8 = in ? *(const bf16x8*)(wb + (size_t)col * I + k) : zero8;
-        acc_b[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b8, x8, acc_b[t], 0, 0, 0);
+        acc[NF + t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b8, x8, acc[NF + t], 0, 0, 0);
       }
     }
   }
-  if (src < 0) return;
 #pragma unroll
-  for (int t = 0; t < 4; ++t)
+  for (int t = 0; t < NA; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) part[wave][t][lane][i] = acc[t][i];
+  __syncthreads();
+  if (wave != 0 || src < 0) return;
+#pragma unroll
+  for (int t = 0; t < NF; ++t)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int col = col0 + t * 16 + lg * 4 + i;
       if (col >= O) continue;
-      const float v = GLU ? activate(acc_a[t][i], act) * acc_b[t][i] : acc_a[t][i];
-      Y[(size_t)place * ldy + col] = (bf16)v;
+      float a = 0.f, b = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        a += part[w][t][lane][i];
+        if (GLU) b += part[w][NF + t][lane][i];
+      }
+      Y[(size_t)place * ldy + col] = (bf16)(GLU ? activate(a, act) * b : a);
     }
+}
+
+// Many pairs: a tile is 128 places, a workgroup of 4 waves computes 128 places x 128 features (GLU: 64 features of both
+// matrices), each wave 64 x 64 as 2 x 2 products of 32 x 32 x 16; tiles of 64 along k go through LDS (rows padded by 16
+// bytes against bank conflicts), double-buffered so that the next tile's loads are in flight while the matrix cores
+// work on the current one.  The rows of X are gathered by the tile's pairs as they are loaded.
+constexpr int TBM = 128, TBN = 128, TBK = 64, TLD = TBK + 8;
+struct MoeTile {
+  bf16 a[TBM][TLD];
+  bf16 w[TBN][TLD];
+};
+template <bool GLU>
+__global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(const bf16* __restrict__ X, long ldx, int top, const int* __restrict__ sorted_pair,
+                                                             const int* __restrict__ tile_expert, const bf16* __restrict__ Wa,
+                                                             const bf16* __restrict__ Wb, long expert_stride, bf16* __restrict__ Y, long ldy,
+                                                             int O, int I, int act) {
+  extern __shared__ __attribute__((aligned(16))) char moe_lds[];
+  MoeTile* tiles = (MoeTile*)moe_lds;               // [2]
+  int* srcs = (int*)(moe_lds + 2 * sizeof(MoeTile));   // [TBM]
+  const int tile = blockIdx.y, e = tile_expert[tile];
+  if (e < 0) return;
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  constexpr int COLS = GLU ? TBN / 2 : TBN;         // features of the result that a workgroup takes
+  const int col0 = blockIdx.x * COLS;
+  if (tid < TBM) {
+    const int pair = sorted_pair[tile * TBM + tid];
+    srcs[tid] = pair < 0 ? -1 : (top > 0 ? pair / top : tile * TBM + tid);
+  }
+  __syncthreads();
+  const bf16* wa = Wa + (size_t)e * expert_stride;
+  const bf16* wb = GLU ? Wb + (size_t)e * expert_stride : nullptr;
+  const int wr = (wave / 2) * 64;
+  // each thread moves 4 chunks of 16 bytes per operand and tile of k; its rows stay the same from tile to tile
+  const bf16* pa[4];
+  const bf16* pw[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = (tid + i * 256) / 8;
+    pa[i] = srcs[r] >= 0 ? X + (size_t)srcs[r] * ldx : nullptr;
+    const int col = col0 + (GLU ? r % COLS : r);
+    pw[i] = col < O ? ((GLU && r >= COLS) ? wb : wa) + (size_t)col * I : nullptr;
+  }
+  uint4 ra[4], rw[4];
+  auto load_global = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int gk = k0 + ((tid + i * 256) % 8) * 8;
+      ra[i] = (pa[i] && gk < I) ? *(const uint4*)(pa[i] + gk) : make_uint4(0, 0, 0, 0);
+      rw[i] = (pw[i] && gk < I) ? *(const uint4*)(pw[i] + gk) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto store_lds = [&](MoeTile& t) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = tid + i * 256, r = c / 8, kc = (c % 8) * 8;
+      *(uint4*)&t.a[r][kc] = ra[i];
+      *(uint4*)&t.w[r][kc] = rw[i];
+    }
+  };
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int m = 0; m < 2; ++m)
+#pragma unroll
+    for (int n = 0; n < 2; ++n)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[m][n][i] = 0.f;
+  // the wave's two column blocks of 32 in the W tile: neighbours (one matrix), or the same features of gate and up
+  const int wc0 = GLU ? (wave % 2) * 32 : (wave % 2) * 64;
+  const int wc1 = GLU ? COLS + wc0 : wc0 + 32;
+  const int n_tiles = (I + TBK - 1) / TBK;
+  load_global(0);
+  store_lds(tiles[0]);
+  __syncthreads();
+  for (int t = 0; t < n_tiles; ++t) {
+    const MoeTile& cur = tiles[t & 1];
+    if (t + 1 < n_tiles) load_global((t + 1) * TBK);
+#pragma unroll
+    for (int kk = 0; kk < TBK / 16; ++kk) {
+      bf16x8 fa[2], fw[2];
+      const int k = kk * 16 + (lane / 32) * 8;
+#pragma unroll
+      for (int m = 0; m < 2; ++m) fa[m] = *(const bf16x8*)&cur.a[wr + m * 32 + lane % 32][k];
+      fw[0] = *(const bf16x8*)&cur.w[wc0 + lane % 32][k];
+      fw[1] = *(const bf16x8*)&cur.w[wc1 + lane % 32][k];
+#pragma unroll
+      for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int n = 0; n < 2; ++n) acc[m][n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[m], fw[n], acc[m][n], 0, 0, 0);
+    }
+    if (t + 1 < n_tiles) {
+      store_lds(tiles[(t + 1) & 1]);   // the other buffer: nobody reads it during this iteration
+      __syncthreads();
+    }
+  }
+  // a lane holds column lane % 32 of a block and its rows (i / 4) * 8 + (lane / 32) * 4 + i % 4
+#pragma unroll
+  for (int m = 0; m < 2; ++m)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int row = wr + m * 32 + (i / 4) * 8 + (lane / 32) * 4 + i % 4;
+      if (srcs[row] < 0) continue;
+      bf16* y = Y + (size_t)(tile * TBM + row) * ldy;
+      if (GLU) {
+        const int col = col0 + wc0 + lane % 32;
+        if (col < O) y[col] = (bf16)(activate(acc[m][0][i], act) * acc[m][1][i]);
+      } else {
+#pragma unroll
+        for (int n = 0; n < 2; ++n) {
+          const int col = col0 + wc0 + n * 32 + lane % 32;
+          if (col < O) y[col] = (bf16)acc[m][n][i];
+        }
+      }
+    }
+}
+constexpr int MOE_TILED_LDS = 2 * (int)sizeof(MoeTile) + TBM * (int)sizeof(int);
+
+template <bool GLU>
+int launch_tiled(const bf16* X, long ldx, int top, const int* sorted_pair, const int* tile_expert, int tiles, const bf16* wa, const bf16* wb,
+                 long stride, bf16* Y, long ldy, int O, int I, int act, hipStream_t stream) {
+  static bool prepared = false;    // (one flag per instantiation)
+  if (!prepared) {
+    hipError_t e = hipFuncSetAttribute((const void*)moe_gemm_tiled_kernel<GLU>, hipFuncAttributeMaxDynamicSharedMemorySize, MOE_TILED_LDS);
+    if (e != hipSuccess) return gibbs_fail("moe_gemm: %s", hipGetErrorString(e));
+    prepared = true;
+  }
+  moe_gemm_tiled_kernel<GLU><<<dim3(ceil_div(O, GLU ? TBN / 2 : TBN), tiles), 256, MOE_TILED_LDS, stream>>>(X, ldx, top, sorted_pair, tile_expert, wa, wb,
+                                                                                                            stride, Y, ldy, O, I, act);
+  return 0;
 }
 
 // ------------------------------------------------------------------------------------------------- combine
@@ -259,8 +412,8 @@ __global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restric
 GIBBS_EXPORT long gibbs_moe_capacity(int n_pairs, int E, int bm) {
   return ((long)n_pairs + (long)E * (bm - 1) + bm - 1) / bm * bm;
 }
-// Tiles of pairs: 16 while the matrices are streamed for few pairs each, 64 beyond.
-GIBBS_EXPORT int gibbs_moe_tile(int n_pairs, int E) { return (long)n_pairs <= 32L * E ? 16 : 64; }
+// Tiles of pairs: 16 while the matrices are streamed for few pairs each (at most 64 an expert on average), 128 beyond.
+GIBBS_EXPORT int gibbs_moe_tile(int n_pairs, int E) { return (long)n_pairs <= 64L * E ? 16 : 128; }
 
 GIBBS_EXPORT int gibbs_moe_route(const void* h, long ldh, int dtype, const float* router, const float* router_bias,
                                  const float* shared_gate, int* chosen, float* weight, float* sgate, int n, int W, int E, int top,
@@ -281,7 +434,7 @@ GIBBS_EXPORT int gibbs_moe_route(const void* h, long ldh, int dtype, const float
 GIBBS_EXPORT int gibbs_moe_group(const int* chosen, int n_pairs, int E, int bm, int* sorted_pair, int* pair_pos, int* tile_expert,
                                  long cap, hipStream_t stream) {
   GIBBS_REQUIRE(chosen && sorted_pair && pair_pos && tile_expert && n_pairs > 0, "moe_group: bad operands pairs=%d", n_pairs);
-  GIBBS_REQUIRE(E > 0 && E <= MOE_MAX_EXPERTS && (bm == 16 || bm == 64), "moe_group: %d experts (at most %d) in tiles of %d (16 or 64)", E, MOE_MAX_EXPERTS, bm);
+  GIBBS_REQUIRE(E > 0 && E <= MOE_MAX_EXPERTS && (bm == 16 || bm == 128), "moe_group: %d experts (at most %d) in tiles of %d (16 or 128)", E, MOE_MAX_EXPERTS, bm);
   GIBBS_REQUIRE(cap >= gibbs_moe_capacity(n_pairs, E, bm) && cap % bm == 0 && cap < (1L << 31), "moe_group: %ld places for %d pairs of %d experts", cap, n_pairs, E);
   moe_group_kernel<<<1, 1024, 0, stream>>>(chosen, n_pairs, E, bm, sorted_pair, pair_pos, tile_expert, (int)cap);
   GIBBS_LAUNCH_STATUS("moe_group");
@@ -294,31 +447,39 @@ GIBBS_EXPORT int gibbs_moe_gemm(const void* X, long ldx, int top, const int* sor
                                 const void* w_a, const void* w_b, void* Y, long ldy, int dtype, int O, int I, int act,
                                 hipStream_t stream) {
   GIBBS_REQUIRE(X && sorted_pair && tile_expert && w_a && Y && O > 0 && I > 0 && ldx >= I && ldy >= O, "moe_gemm: bad operands O=%d I=%d", O, I);
-  GIBBS_REQUIRE((bm == 16 || bm == 64) && cap > 0 && cap % bm == 0 && cap / bm <= 65535, "moe_gemm: %ld places in tiles of %d", cap, bm);
+  GIBBS_REQUIRE((bm == 16 || bm == 128) && cap > 0 && cap % bm == 0 && cap / bm <= 65535, "moe_gemm: %ld places in tiles of %d", cap, bm);
   GIBBS_REQUIRE(top >= 0 && act >= 0 && act < ACT_COUNT, "moe_gemm: bad choice count or activation");
   const long stride = (long)O * I;
   const int tiles = (int)(cap / bm);
 #define MOE_PLAIN(T, BM, GLU)                                                                                                     \
   moe_gemm_plain_kernel<T, BM, GLU><<<dim3(ceil_div(O, 64), tiles), 256, 0, stream>>>((const T*)X, ldx, top, sorted_pair, tile_expert, \
                                                                                      (const T*)w_a, (const T*)w_b, stride, (T*)Y, ldy, O, I, act)
-#define MOE_MFMA(BM, GLU)                                                                                                          \
-  moe_gemm_mfma_kernel<BM, GLU><<<dim3(ceil_div(O, BM == 64 ? 64 : 256), tiles), 256, 0, stream>>>(                                 \
-      (const bf16*)X, ldx, top, sorted_pair, tile_expert, (const bf16*)w_a, (const bf16*)w_b, stride, (bf16*)Y, ldy, O, I, act)
-#define MOE_PICK(LAUNCH, ...)                                        \
-  do {                                                               \
-    if (bm == 64) { if (w_b) LAUNCH(__VA_ARGS__ 64, true); else LAUNCH(__VA_ARGS__ 64, false); } \
-    else { if (w_b) LAUNCH(__VA_ARGS__ 16, true); else LAUNCH(__VA_ARGS__ 16, false); }          \
+#define MOE_PLAIN_ANY(T)                                                                  \
+  do {                                                                                    \
+    if (bm == 128) { if (w_b) MOE_PLAIN(T, 128, true); else MOE_PLAIN(T, 128, false); }    \
+    else { if (w_b) MOE_PLAIN(T, 16, true); else MOE_PLAIN(T, 16, false); }                \
   } while (0)
   if (dtype == GIBBS_F32) {
-    MOE_PICK(MOE_PLAIN, float,);
+    MOE_PLAIN_ANY(float);
   } else if (dtype == GIBBS_BF16) {
     const bool aligned = I % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)X % 16) == 0 && ((uintptr_t)w_a % 16) == 0 && ((uintptr_t)w_b % 16) == 0;
-    if (aligned) MOE_PICK(MOE_MFMA,); else MOE_PICK(MOE_PLAIN, bf16,);
+    if (!aligned) {
+      MOE_PLAIN_ANY(bf16);
+    } else if (bm == 128) {
+      if (w_b ? launch_tiled<true>((const bf16*)X, ldx, top, sorted_pair, tile_expert, tiles, (const bf16*)w_a, (const bf16*)w_b, stride, (bf16*)Y, ldy, O, I, act, stream)
+              : launch_tiled<false>((const bf16*)X, ldx, top, sorted_pair, tile_expert, tiles, (const bf16*)w_a, nullptr, stride, (bf16*)Y, ldy, O, I, act, stream))
+        return 1;
+    } else if (w_b) {
+      moe_gemm_few_kernel<true><<<dim3(ceil_div(O, 32), tiles), 256, 0, stream>>>((const bf16*)X, ldx, top, sorted_pair, tile_expert, (const bf16*)w_a,
+                                                                                 (const bf16*)w_b, stride, (bf16*)Y, ldy, O, I, act);
+    } else {
+      moe_gemm_few_kernel<false><<<dim3(ceil_div(O, 32), tiles), 256, 0, stream>>>((const bf16*)X, ldx, top, sorted_pair, tile_expert, (const bf16*)w_a,
+                                                                                  nullptr, stride, (bf16*)Y, ldy, O, I, act);
+    }
   } else {
     return gibbs_fail("moe_gemm: unknown dtype %d", dtype);
   }
-#undef MOE_PICK
-#undef MOE_MFMA
+#undef MOE_PLAIN_ANY
 #undef MOE_PLAIN
   GIBBS_LAUNCH_STATUS("moe_gemm");
 }

@@ -332,7 +332,7 @@ def test_experts_route_group_products_and_combine(case):
     lib = library()
     pairs = n * top
     bm = lib.gibbs_moe_tile(pairs, E)
-    assert bm == (64 if n == 300 else 16)
+    assert bm == (128 if n == 300 else 16)
     cap = lib.gibbs_moe_capacity(pairs, E, bm)
     sorted_pair = torch.empty(cap, dtype=torch.int32, device="cuda")
     place = torch.empty(pairs, dtype=torch.int32, device="cuda")
