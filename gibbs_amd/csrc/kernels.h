@@ -15,6 +15,8 @@ int gibbs_rmsnorm_rows(const void* in, int parts, long part_stride, const float*
                        int hidden, hipStream_t stream);
 int gibbs_rmsnorm_rows_add(float* x, const void* in, int parts, long part_stride, const float* gain, float eps, int dtype, int n,
                            int hidden, hipStream_t stream);
+int gibbs_rmsnorm_rows_add_norm(float* x, const void* in, int parts, long part_stride, const float* gain_d, float eps_d,
+                                const float* gain_n, float eps_n, void* out, int dtype, int n, int hidden, hipStream_t stream);
 int gibbs_glu_clamped(const void* gu, void* out, int dtype, int n, int F, float alpha, float limit, hipStream_t stream);
 int gibbs_attention_plain_general(const void* q, const void* kpages, const void* vpages, void* out, int dtype, const int* pos,
                                   const int* row_req, const int* table, int max_pages, int page_size, int num_pages, int n_rows,

@@ -25,6 +25,35 @@ namespace {
 constexpr int MOE_MAX_EXPERTS = 1024;
 
 // ------------------------------------------------------------------------------------------------- route
+// 4 neighbouring values of a row as float32 (16-byte or 8-byte loads)
+__device__ __forceinline__ float4 load4f(const float* p) { return *(const float4*)p; }
+__device__ __forceinline__ float4 load4f(const bf16* p) {
+  const uint2 raw = *(const uint2*)p;
+  return make_float4(__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u), __uint_as_float(raw.y << 16),
+                     __uint_as_float(raw.y & 0xffff0000u));
+}
+__device__ __forceinline__ void store4f(float* p, float4 v) { *(float4*)p = v; }
+__device__ __forceinline__ void store4f(bf16* p, float4 v) {
+  union { bf16 h[4]; uint2 u; } o;
+  o.h[0] = (bf16)v.x; o.h[1] = (bf16)v.y; o.h[2] = (bf16)v.z; o.h[3] = (bf16)v.w;
+  *(uint2*)p = o.u;
+}
+// One wave's inner product of a row with a float32 vector; `vec`: the width is a multiple of 4 and both are aligned, so a
+// lane takes 4 neighbouring values at a time (the order of the additions depends on the width alone).
+template <typename T>
+__device__ __forceinline__ float wave_dot(const T* __restrict__ row, const float* __restrict__ w, int W, int lane, bool vec) {
+  float s = 0.f;
+  if (vec) {
+    for (int k = lane * 4; k < W; k += WAVE * 4) {
+      const float4 a = load4f(row + k), b = *(const float4*)(w + k);
+      s = fmaf(a.x, b.x, s); s = fmaf(a.y, b.y, s); s = fmaf(a.z, b.z, s); s = fmaf(a.w, b.w, s);
+    }
+  } else {
+    for (int k = lane; k < W; k += WAVE) s = fmaf(to_float(row[k]), w[k], s);
+  }
+  return wave_sum(s);
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, long ldh, const float* __restrict__ router,
                                                         const float* __restrict__ router_bias, const float* __restrict__ shared_gate,
@@ -33,17 +62,13 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
   extern __shared__ float z[];   // [E]
   const int n = blockIdx.x, wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, n_waves = blockDim.x / WAVE;
   const T* row = h + (size_t)n * ldh;
+  const bool vec = W % 4 == 0 && ldh % 4 == 0 && ((uintptr_t)h % 16) == 0 && ((uintptr_t)router % 16) == 0 && ((uintptr_t)shared_gate % 16) == 0;
   for (int e = wave; e < E; e += n_waves) {
-    const float* w = router + (size_t)e * W;
-    float s = 0.f;
-    for (int k = lane; k < W; k += WAVE) s = fmaf(to_float(row[k]), w[k], s);
-    s = wave_sum(s);
+    const float s = wave_dot(row, router + (size_t)e * W, W, lane, vec);
     if (lane == 0) z[e] = s + (router_bias ? router_bias[e] : 0.f);
   }
-  if (shared_gate && wave == 0) {
-    float s = 0.f;
-    for (int k = lane; k < W; k += WAVE) s = fmaf(to_float(row[k]), shared_gate[k], s);
-    s = wave_sum(s);
+  if (shared_gate && wave == n_waves - 1) {
+    const float s = wave_dot(row, shared_gate, W, lane, vec);
     if (lane == 0) sgate[n] = 1.0f / (1.0f + expf(-s));
   }
   __syncthreads();
@@ -394,11 +419,41 @@ int launch_tiled(const bf16* X, long ldx, int top, const int* sorted_pair, const
 }
 
 // ------------------------------------------------------------------------------------------------- combine
-template <typename T>
+template <typename T, bool VEC>
 __global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restrict__ pair_pos, const float* __restrict__ weight,
                                    const T* __restrict__ shared, const float* __restrict__ sgate, T* __restrict__ out, int top, int W) {
+  constexpr int MOST = 8;      // choices whose places and weights a thread keeps in registers
   const int n = blockIdx.x;
   const float g = shared ? (sgate ? sgate[n] : 1.0f) : 0.f;
+  size_t at[MOST];
+  float w[MOST];
+#pragma unroll
+  for (int s = 0; s < MOST; ++s) {
+    at[s] = s < top ? (size_t)pair_pos[(size_t)n * top + s] * W : 0;
+    w[s] = s < top ? weight[(size_t)n * top + s] : 0.f;
+  }
+  if (VEC) {
+    for (int c = threadIdx.x * 4; c < W; c += blockDim.x * 4) {
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int s = 0; s < MOST; ++s)
+        if (s < top) {
+          const float4 r = load4f(y + at[s] + c);
+          v.x = fmaf(w[s], r.x, v.x); v.y = fmaf(w[s], r.y, v.y); v.z = fmaf(w[s], r.z, v.z); v.w = fmaf(w[s], r.w, v.w);
+        }
+      for (int s = MOST; s < top; ++s) {
+        const float ws = weight[(size_t)n * top + s];
+        const float4 r = load4f(y + (size_t)pair_pos[(size_t)n * top + s] * W + c);
+        v.x = fmaf(ws, r.x, v.x); v.y = fmaf(ws, r.y, v.y); v.z = fmaf(ws, r.z, v.z); v.w = fmaf(ws, r.w, v.w);
+      }
+      if (shared) {
+        const float4 r = load4f(shared + (size_t)n * W + c);
+        v.x = fmaf(g, r.x, v.x); v.y = fmaf(g, r.y, v.y); v.z = fmaf(g, r.z, v.z); v.w = fmaf(g, r.w, v.w);
+      }
+      store4f(out + (size_t)n * W + c, v);
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     float v = 0.f;
     for (int s = 0; s < top; ++s) v = fmaf(weight[(size_t)n * top + s], to_float(y[(size_t)pair_pos[(size_t)n * top + s] * W + c]), v);
@@ -488,12 +543,15 @@ GIBBS_EXPORT int gibbs_moe_gemm(const void* X, long ldx, int top, const int* sor
 GIBBS_EXPORT int gibbs_moe_combine(const void* y, const int* pair_pos, const float* weight, const void* shared, const float* sgate,
                                    void* out, int dtype, int n, int top, int W, hipStream_t stream) {
   GIBBS_REQUIRE(y && pair_pos && weight && out && n > 0 && top > 0 && W > 0, "moe_combine: bad operands n=%d top=%d width=%d", n, top, W);
-  const int threads = W >= 1024 ? 256 : 64;
-  if (dtype == GIBBS_F32)
-    moe_combine_kernel<float><<<n, threads, 0, stream>>>((const float*)y, pair_pos, weight, (const float*)shared, sgate, (float*)out, top, W);
-  else if (dtype == GIBBS_BF16)
-    moe_combine_kernel<bf16><<<n, threads, 0, stream>>>((const bf16*)y, pair_pos, weight, (const bf16*)shared, sgate, (bf16*)out, top, W);
-  else
+  const size_t bytes = dtype == GIBBS_F32 ? 16 : 8;
+  const bool vec = W % 4 == 0 && ((uintptr_t)y % bytes) == 0 && ((uintptr_t)shared % bytes) == 0 && ((uintptr_t)out % bytes) == 0;
+  const int threads = vec ? (W >= 4096 ? 1024 : (W >= 1024 ? 256 : 64)) : (W >= 1024 ? 256 : 64);
+#define MOE_COMBINE(T, V) moe_combine_kernel<T, V><<<n, threads, 0, stream>>>((const T*)y, pair_pos, weight, (const T*)shared, sgate, (T*)out, top, W)
+  if (dtype == GIBBS_F32) {
+    if (vec) MOE_COMBINE(float, true); else MOE_COMBINE(float, false);
+  } else if (dtype == GIBBS_BF16) {
+    if (vec) MOE_COMBINE(bf16, true); else MOE_COMBINE(bf16, false);
+  } else
     return gibbs_fail("moe_combine: unknown dtype %d", dtype);
   GIBBS_LAUNCH_STATUS("moe_combine");
 }

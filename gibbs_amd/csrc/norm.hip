@@ -252,10 +252,103 @@ __global__ void rmsnorm_rows_add_kernel(float* __restrict__ x, const void* __res
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) x[at + i] += gain ? value(i) * scale * gain[i] : value(i) * scale;
 }
 
+// A sublayer's boundary in one pass: x += v * rsqrt(mean(v^2) + eps_d) * gain_d, v the sum of the `parts` partial sums of a
+// part's result (one, in the activation type, or several in float32); and, with `out`, out = x * rsqrt(mean(x^2) + eps_n) *
+// gain_n of the new x (the next sublayer's norm).  A thread keeps its elements of the row in registers between the sums and
+// the scalings: 16-byte accesses, hidden sizes in steps of 4 up to 4 * CHUNKS * blockDim.  Sums, roots and x are float32.
+template <typename T, int CHUNKS>
+__global__ void rows_add_norm_vec_kernel(float* __restrict__ x, const void* __restrict__ in, int parts, size_t part_stride,
+                                         const float* __restrict__ gain_d, float eps_d, const float* __restrict__ gain_n, float eps_n,
+                                         T* __restrict__ out, int hidden) {
+  __shared__ float scratch[16];
+  const size_t at = (size_t)blockIdx.x * hidden;
+  float4 v[CHUNKS], xv[CHUNKS];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int i = (c * blockDim.x + threadIdx.x) * 4;
+    v[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (i < hidden) {
+      xv[c] = *(const float4*)(x + at + i);
+      if (parts == 1) {
+        v[c] = load4((const T*)in + at + i);
+      } else {
+        for (int s = 0; s < parts; ++s) {
+          const float4 d = *(const float4*)((const float*)in + s * part_stride + at + i);
+          v[c].x += d.x; v[c].y += d.y; v[c].z += d.z; v[c].w += d.w;
+        }
+      }
+      ss += v[c].x * v[c].x + v[c].y * v[c].y + v[c].z * v[c].z + v[c].w * v[c].w;
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float scale = 1.0f / sqrtf(ss / (float)hidden + eps_d);
+  float sx = 0.f;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int i = (c * blockDim.x + threadIdx.x) * 4;
+    if (i < hidden) {
+      float4 g = make_float4(1.f, 1.f, 1.f, 1.f);
+      if (gain_d) g = *(const float4*)(gain_d + i);
+      xv[c].x += v[c].x * scale * g.x; xv[c].y += v[c].y * scale * g.y; xv[c].z += v[c].z * scale * g.z; xv[c].w += v[c].w * scale * g.w;
+      *(float4*)(x + at + i) = xv[c];
+      sx += xv[c].x * xv[c].x + xv[c].y * xv[c].y + xv[c].z * xv[c].z + xv[c].w * xv[c].w;
+    }
+  }
+  if (!out) return;
+  sx = block_sum(sx, scratch);
+  const float scale_n = 1.0f / sqrtf(sx / (float)hidden + eps_n);
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int i = (c * blockDim.x + threadIdx.x) * 4;
+    if (i < hidden) {
+      float4 g = make_float4(1.f, 1.f, 1.f, 1.f);
+      if (gain_n) g = *(const float4*)(gain_n + i);
+      store4(out + at + i, make_float4(xv[c].x * scale_n * g.x, xv[c].y * scale_n * g.y, xv[c].z * scale_n * g.z, xv[c].w * scale_n * g.w));
+    }
+  }
+}
+
+template <typename T>
+bool launch_rows_add_norm(float* x, const void* in, int parts, long part_stride, const float* gain_d, float eps_d, const float* gain_n,
+                          float eps_n, T* out, int n, int hidden, hipStream_t stream) {
+  const uintptr_t vec = parts == 1 ? 4 * sizeof(T) : 16;
+  if (hidden % 4 || ((uintptr_t)x % 16) || ((uintptr_t)in % vec) || (parts > 1 && part_stride % 4) || (gain_d && ((uintptr_t)gain_d % 16)) ||
+      (gain_n && ((uintptr_t)gain_n % 16)) || (out && ((uintptr_t)out % (4 * sizeof(T)))))
+    return false;
+  // (few rows: wide workgroups, every load of the row in flight at once)
+  const int threads = hidden >= 4096 ? 1024 : (hidden >= 2048 ? 512 : (hidden >= 512 ? 256 : 64));
+  const int chunks = ceil_div(hidden, 4 * threads);
+#define GIBBS_ROWS_ADD_NORM(C) rows_add_norm_vec_kernel<T, C><<<n, threads, 0, stream>>>(x, in, parts, (size_t)part_stride, gain_d, eps_d, gain_n, eps_n, out, hidden)
+  if (chunks == 1) GIBBS_ROWS_ADD_NORM(1);
+  else if (chunks == 2) GIBBS_ROWS_ADD_NORM(2);
+  else if (chunks <= 4) GIBBS_ROWS_ADD_NORM(4);
+  else return false;
+#undef GIBBS_ROWS_ADD_NORM
+  return true;
+}
+
+// x += norm(in) (gain_d, eps_d) and out = norm(x) (gain_n, eps_n) of all n rows in one kernel.  Returns 0 when it was queued,
+// -1 when the sizes or addresses do not allow it (nothing was queued: the caller runs the two passes), 1 on an error.
+GIBBS_EXPORT int gibbs_rmsnorm_rows_add_norm(float* x, const void* in, int parts, long part_stride, const float* gain_d, float eps_d,
+                                             const float* gain_n, float eps_n, void* out, int dtype, int n, int hidden, hipStream_t stream) {
+  GIBBS_REQUIRE(x && in && out && n >= 0 && hidden > 0 && parts >= 1, "rmsnorm_rows_add_norm: bad sizes n=%d hidden=%d parts=%d", n, hidden, parts);
+  if (n == 0) return 0;
+  bool queued;
+  if (dtype == GIBBS_F32) queued = launch_rows_add_norm<float>(x, in, parts, part_stride, gain_d, eps_d, gain_n, eps_n, (float*)out, n, hidden, stream);
+  else if (dtype == GIBBS_BF16) queued = launch_rows_add_norm<bf16>(x, in, parts, part_stride, gain_d, eps_d, gain_n, eps_n, (bf16*)out, n, hidden, stream);
+  else return gibbs_fail("rmsnorm_rows_add_norm: unknown dtype %d", dtype);
+  if (!queued) return -1;
+  GIBBS_LAUNCH_STATUS("rmsnorm_rows_add_norm");
+}
+
 GIBBS_EXPORT int gibbs_rmsnorm_rows_add(float* x, const void* in, int parts, long part_stride, const float* gain, float eps, int dtype,
                                         int n, int hidden, hipStream_t stream) {
   GIBBS_REQUIRE(x && in && n >= 0 && hidden > 0 && parts >= 1, "rmsnorm_rows_add: bad sizes n=%d hidden=%d parts=%d", n, hidden, parts);
   if (n == 0) return 0;
+  if ((dtype == GIBBS_F32 && launch_rows_add_norm<float>(x, in, parts, part_stride, gain, eps, nullptr, 0.f, nullptr, n, hidden, stream)) ||
+      (dtype == GIBBS_BF16 && launch_rows_add_norm<bf16>(x, in, parts, part_stride, gain, eps, nullptr, 0.f, nullptr, n, hidden, stream)))
+    GIBBS_LAUNCH_STATUS("rmsnorm_rows_add");
   const int threads = hidden >= 2048 ? 512 : (hidden >= 512 ? 256 : 64);
   if (dtype == GIBBS_F32)
     rmsnorm_rows_add_kernel<float><<<n, threads, 0, stream>>>(x, in, parts, (size_t)part_stride, gain, eps, hidden);

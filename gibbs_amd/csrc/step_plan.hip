@@ -270,6 +270,8 @@ struct NormPart {
   // the norm of a weighted sum of several residual streams x [streams][N][hidden] (coef null: their plain sum), of all
   // rows or of `rows`; the streams are not touched
   virtual void* run_streams(Exec& e, const float* x, int streams, const float* coef, const int* rows, int n_out) const;
+  // a plain RMS norm with its gain (null: none) and eps, for kernels that apply it beside their own work
+  virtual bool plain_rms(const float** gain, float* eps) const { return false; }
   // a norm that the streams' kernels apply themselves: its kind there (0 root mean square, 1 layer norm) and operands
   virtual bool for_streams(int* kind, const float** gain, const float** bias, float* eps) const { return false; }
 };
@@ -415,6 +417,10 @@ struct RmsNorm : NormPart {
   bool folded_rms(float* e) const override {
     *e = eps;
     return gain == nullptr;
+  }
+  bool plain_rms(const float** g, float* e) const override {
+    *g = gain; *e = eps;
+    return true;
   }
   bool add_normed(Exec& e, float* x, Pending delta) const override {
     const int N = e.a.n_rows, H = e.p.hidden;
@@ -721,13 +727,19 @@ struct GluBody : Body {
   }
   Pending general(Exec& e, void* h) const override {
     const int N = e.a.n_rows;
-    void* gu = e.linear(h, gate_up, N, false, false, false, nullptr);
     void* y = e.take((long)N * F * e.esize);
-    if (act == ACT_CLAMPED)
-      RUN(e, gibbs_glu_clamped(gu, y, e.p.dtype, N, F, alpha, limit, e.a.stream));
-    else
-      RUN(e, gibbs_glu(gu, y, e.p.dtype, N, F, act, e.a.stream));
-    e.give(gu);
+    if (e.few_rows && fusable(false)) {
+      // few rows: the gated product is the few-row kernel's epilogue (gate and up stay float32 until the product)
+      RUN(e, gibbs_skinny_glu_general(h, gate_up_packed2 ? gate_up_packed2 : gate_up.w, y, N, F, gate_up.I, gate_up.I, gate_up_packed2 ? 0 : gate_up.I, F,
+                                      0, 0.f, act, alpha, limit, e.a.stream));
+    } else {
+      void* gu = e.linear(h, gate_up, N, false, false, false, nullptr);
+      if (act == ACT_CLAMPED)
+        RUN(e, gibbs_glu_clamped(gu, y, e.p.dtype, N, F, alpha, limit, e.a.stream));
+      else
+        RUN(e, gibbs_glu(gu, y, e.p.dtype, N, F, act, e.a.stream));
+      e.give(gu);
+    }
     Pending delta;
     delta.data = e.linear(y, down, N, false, true, true, &delta.parts);
     e.give(y);
@@ -959,10 +971,14 @@ struct MoeBody : Body {
     e.give(tile_expert);
     void* shared = nullptr;
     if (shared_gate_up.w) {
-      void* gu = e.linear(h, shared_gate_up, N, false, false, false, nullptr);
       void* sy = e.take((long)N * SF * e.esize);
-      RUN(e, gibbs_glu(gu, sy, e.p.dtype, N, SF, shared_act, e.a.stream));
-      e.give(gu);
+      if (e.few_rows && W % 8 == 0 && SF % 8 == 0) {
+        RUN(e, gibbs_skinny_glu_general(h, shared_gate_up.w, sy, N, SF, W, W, W, SF, 0, 0.f, shared_act, 0.f, 0.f, e.a.stream));
+      } else {
+        void* gu = e.linear(h, shared_gate_up, N, false, false, false, nullptr);
+        RUN(e, gibbs_glu(gu, sy, e.p.dtype, N, SF, shared_act, e.a.stream));
+        e.give(gu);
+      }
       shared = e.linear(sy, shared_down, N, false, false, false, nullptr);
       e.give(sy);
     }
@@ -1056,7 +1072,33 @@ void Exec::run() {
         deltas[op.result] = p.norms[op.norm]->run_on(*this, deltas[op.value]);
         deltas[op.value] = Pending{};
         break;
-      case Plan::OP_ADD_NORMED:
+      case Plan::OP_ADD_NORMED: {
+        // x += norm(delta) and the norm of the new x that the next operation asks for, in one kernel: a sublayer's
+        // boundary (both norms plain RMS norms, nothing pending, sizes that the kernel takes)
+        const Plan::Op* next = i + 1 < last && p.ops[i + 1].kind == Plan::OP_NORM ? &p.ops[i + 1] : nullptr;
+        const float *gain_d = nullptr, *gain_n = nullptr;
+        float eps_d = 0.f, eps_n = 0.f;
+        Pending& d = deltas[op.value];
+        if (next && pending.parts == 0 && d.data && p.norms[op.norm]->plain_rms(&gain_d, &eps_d) && p.norms[next->norm]->plain_rms(&gain_n, &eps_n)) {
+          void* out = take((long)N * H * esize);
+          int fused = -1;
+          if (!dry && status == 0) {
+            fused = gibbs_rmsnorm_rows_add_norm(x, d.data, std::max(d.parts, 1), (long)N * H, gain_d, eps_d, gain_n, eps_n, out, p.dtype, N, H, a.stream);
+            if (fused > 0) status = 1;
+          } else if (H % 4 == 0 && H <= 16384) {
+            fused = 0;      // (a dry run: the same buffers as the real one will take)
+          }
+          if (fused == 0) {
+            give(d.data);
+            d = Pending{};
+            give(mirror);
+            mirror = nullptr;
+            rows[next->result] = out;
+            ++i;
+            break;
+          }
+          give(out);
+        }
         // (what is pending stays pending: additions into x commute, and the next norm still takes it on its way)
         if (p.norms[op.norm]->add_normed(*this, x, deltas[op.value])) {
           deltas[op.value] = Pending{};
@@ -1068,6 +1110,7 @@ void Exec::run() {
           deltas[op.value] = Pending{};
         }
         break;
+      }
       case Plan::OP_REINJECT:
         settle(x, pending);
         if (!embedded) { if (!status) status = gibbs_fail("step: the embedding's output is added again, but the caller brought the rows"); break; }

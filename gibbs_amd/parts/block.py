@@ -126,6 +126,10 @@ class SandwichBlock(Block):
         if self.mult != 1.0:
             for norm in [self.norm1b] + ([self.norm2b] if self.has_ffn else []):
                 norm.gain = (norm.gain * self.mult).contiguous()
+        if rt.act_dtype == torch.bfloat16:       # (tile-ordered copies for the few-row products of decode steps)
+            self.mixer.pack_matrices()
+            if self.has_ffn:
+                self.ffn.pack_matrices()
 
     def emit(self, plan, caches) -> None:
         subs = [(self.norm1, lambda: self.mixer.emit(plan, caches["mixer"]), self.norm1b)]
