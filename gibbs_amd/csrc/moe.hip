@@ -20,6 +20,7 @@
 // pairs beyond (128 x 128 x 64 through LDS, double-buffered, as the framework's tiled product).
 #include "common.h"
 #include "activation.h"
+#include <algorithm>
 
 namespace {
 constexpr int MOE_MAX_EXPERTS = 1024;
@@ -44,7 +45,19 @@ template <typename T>
 __device__ __forceinline__ float wave_dot(const T* __restrict__ row, const float* __restrict__ w, int W, int lane, bool vec) {
   float s = 0.f;
   if (vec) {
-    for (int k = lane * 4; k < W; k += WAVE * 4) {
+    // (four steps at a time: their loads are asked for together)
+    int k = lane * 4;
+    for (; k + 3 * WAVE * 4 < W; k += 4 * WAVE * 4) {
+      float4 a[4], b[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        a[u] = load4f(row + k + u * WAVE * 4);
+        b[u] = *(const float4*)(w + k + u * WAVE * 4);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) { s = fmaf(a[u].x, b[u].x, s); s = fmaf(a[u].y, b[u].y, s); s = fmaf(a[u].z, b[u].z, s); s = fmaf(a[u].w, b[u].w, s); }
+    }
+    for (; k < W; k += WAVE * 4) {
       const float4 a = load4f(row + k), b = *(const float4*)(w + k);
       s = fmaf(a.x, b.x, s); s = fmaf(a.y, b.y, s); s = fmaf(a.z, b.z, s); s = fmaf(a.w, b.w, s);
     }
@@ -55,7 +68,7 @@ __device__ __forceinline__ float wave_dot(const T* __restrict__ row, const float
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, long ldh, const float* __restrict__ router,
+__global__ __launch_bounds__(1024) void moe_route_kernel(const T* __restrict__ h, long ldh, const float* __restrict__ router,
                                                         const float* __restrict__ router_bias, const float* __restrict__ shared_gate,
                                                         int* __restrict__ chosen, float* __restrict__ weight, float* __restrict__ sgate,
                                                         int W, int E, int top) {
@@ -477,10 +490,12 @@ GIBBS_EXPORT int gibbs_moe_route(const void* h, long ldh, int dtype, const float
   GIBBS_REQUIRE(E > 0 && E <= MOE_MAX_EXPERTS && top > 0 && top <= E, "moe_route: %d of %d experts (at most %d)", top, E, MOE_MAX_EXPERTS);
   GIBBS_REQUIRE(!shared_gate || sgate, "moe_route: a shared expert's gate needs its output");
   const size_t lds = (size_t)E * sizeof(float);
+  // few rows: a wave per expert (and one for the shared expert's gate) up to 16 waves; many rows fill the chip with 4
+  const int threads = n >= 512 ? 256 : WAVE * std::min(16, std::max(4, E + 1));
   if (dtype == GIBBS_F32)
-    moe_route_kernel<float><<<n, 256, lds, stream>>>((const float*)h, ldh, router, router_bias, shared_gate, chosen, weight, sgate, W, E, top);
+    moe_route_kernel<float><<<n, threads, lds, stream>>>((const float*)h, ldh, router, router_bias, shared_gate, chosen, weight, sgate, W, E, top);
   else if (dtype == GIBBS_BF16)
-    moe_route_kernel<bf16><<<n, 256, lds, stream>>>((const bf16*)h, ldh, router, router_bias, shared_gate, chosen, weight, sgate, W, E, top);
+    moe_route_kernel<bf16><<<n, threads, lds, stream>>>((const bf16*)h, ldh, router, router_bias, shared_gate, chosen, weight, sgate, W, E, top);
   else
     return gibbs_fail("moe_route: unknown dtype %d", dtype);
   GIBBS_LAUNCH_STATUS("moe_route");

@@ -93,6 +93,109 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(T* __restrict__ rows, 
   }
   for (int e = 2 * half + lane; e < size; e += WAVE) put(e, value(e));
 }
+
+// The same for bfloat16 rows whose sizes are multiples of 8 (heads, values, published values) and whose rotated part is
+// a multiple of 16 in half-split pairs: a thread takes 8 neighbouring channels with 16-byte accesses, or, inside the rotated
+// part, the 8 channels j .. j + 7 and their partners j + rot/2 ..; the threads are numbered over all (row, item) of the step,
+// so that a wave is full whatever the head size.
+__device__ __forceinline__ void unpack_bf16x8(const uint4& raw, float* f) { unpack8(raw, f); }
+__device__ __forceinline__ uint4 pack_bf16x8(const float* f) {
+  union { bf16 h[8]; uint4 u; } o;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) o.h[i] = (bf16)f[i];
+  return o.u;
+}
+__global__ __launch_bounds__(256) void qkv_prepare_bf16x8_kernel(bf16* __restrict__ rows, bf16* __restrict__ kpages, bf16* __restrict__ vpages,
+                                                                 bf16* __restrict__ keep, QkvPrepareArgs a, int n_rows) {
+  const int half = a.inv_freq ? a.rot / 2 : 0;
+  const int per_qk = half / 8 + (a.hd - 2 * half) / 8, per_v = a.vd / 8;
+  const int per_row = (a.nh + a.nkv) * per_qk + a.nkv * per_v;
+  const unsigned item = blockIdx.x * blockDim.x + threadIdx.x;
+  if (item >= (unsigned)n_rows * (unsigned)per_row) return;
+  const int n = (int)(item / (unsigned)per_row);
+  int it = (int)(item % (unsigned)per_row);
+  const int p = a.pos[n];
+  bf16* row = rows + (size_t)n * a.ld;
+  const bool is_v = it >= (a.nh + a.nkv) * per_qk;
+  int head, sub;
+  if (is_v) {
+    it -= (a.nh + a.nkv) * per_qk;
+    head = it / per_v;
+    sub = it % per_v;
+  } else {
+    head = it / per_qk;
+    sub = it % per_qk;
+  }
+  const bool is_q = !is_v && head < a.nh;
+  const int g = is_v ? head : (is_q ? head : head - a.nh);
+  const long off = is_v ? (long)(a.nh + a.nkv) * a.hd + (long)g * a.vd : (long)head * a.hd;
+  const int size = is_v ? a.vd : a.hd;
+  bf16* page_dst = nullptr;
+  if (!is_q && kpages) {
+    const int page = a.table[(size_t)a.row_req[n] * a.max_pages + p / a.page_size];
+    if (page >= 0 && page < a.num_pages)
+      page_dst = (is_v ? vpages : kpages) + (((size_t)page * a.nkv + g) * a.page_size + p % a.page_size) * size;
+  }
+  bf16* src = row + off;
+  const float* bias = a.bias ? a.bias + off : nullptr;
+  auto load = [&](int e0, float* f) {
+    unpack_bf16x8(*(const uint4*)(src + e0), f);
+    if (bias) {
+      const float4 b0 = *(const float4*)(bias + e0), b1 = *(const float4*)(bias + e0 + 4);
+      f[0] += b0.x; f[1] += b0.y; f[2] += b0.z; f[3] += b0.w; f[4] += b1.x; f[5] += b1.y; f[6] += b1.z; f[7] += b1.w;
+    }
+  };
+  auto put = [&](int e0, const float* f) {
+    const uint4 r = pack_bf16x8(f);
+    *(uint4*)(src + e0) = r;
+    if (page_dst) *(uint4*)(page_dst + e0) = r;
+  };
+  if (is_v) {
+    const int e0 = sub * 8;
+    float v[8];
+    load(e0, v);
+    if (a.keep_mode != KEEP_NONE && e0 < a.vt) {
+      bf16* kept = keep + ((size_t)n * a.nkv + g) * a.vt + e0;
+      if (a.keep_mode == KEEP_MIX) {
+        const float lam = *a.lambda;
+        float o[8];
+        unpack_bf16x8(*(const uint4*)kept, o);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (1.0f - lam) * v[i] + lam * o[i];
+      } else {
+        *(uint4*)kept = pack_bf16x8(v);
+      }
+    }
+    put(e0, v);
+    return;
+  }
+  if (sub >= half / 8) {   // channels behind the rotated part pass
+    const int e0 = 2 * half + (sub - half / 8) * 8;
+    float v[8];
+    load(e0, v);
+    put(e0, v);
+    return;
+  }
+  const int j0 = sub * 8;
+  float x0[8], x1[8], y0[8], y1[8];
+  load(j0, x0);
+  load(j0 + half, x1);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    float c, s;
+    if (a.cs_table && p < a.table_len) {
+      const float2 cs = a.cs_table[(size_t)p * half + j0 + i];
+      c = cs.x;
+      s = cs.y;
+    } else {
+      rope_cos_sin((float)p * a.inv_freq[j0 + i], &c, &s);
+    }
+    y0[i] = x0[i] * c - x1[i] * s;
+    y1[i] = x1[i] * c + x0[i] * s;
+  }
+  put(j0, y0);
+  put(j0 + half, y1);
+}
 }  // namespace
 
 // keep_mode: 0 none, 1 the values are published into `keep`, 2 `keep` is mixed into the values with *lambda.
@@ -109,6 +212,17 @@ GIBBS_EXPORT int gibbs_qkv_prepare(void* rows, long ld, void* kpages, void* vpag
                 "qkv_prepare: value mixing needs the published values and its weight");
   QkvPrepareArgs a{bias, inv_freq, inv_freq ? rot : 0, variant, (const float2*)cs_table, cs_table && inv_freq ? table_len : 0, lambda, keep_mode, vt,
                    pos, row_req, table, max_pages, page_size, num_pages, nh, nkv, hd, vd, ld};
+  const bool x8 = dtype == GIBBS_BF16 && hd % 8 == 0 && vd % 8 == 0 && ld % 8 == 0 && ((uintptr_t)rows % 16) == 0 && (!inv_freq || (variant == ROPE_HALF_SPLIT && rot % 16 == 0)) &&
+                  (!bias || ((uintptr_t)bias % 16) == 0) && (keep_mode == KEEP_NONE || (vt % 8 == 0 && ((uintptr_t)keep % 16) == 0)) &&
+                  (!kpages || (((uintptr_t)kpages % 16) == 0 && ((uintptr_t)vpages % 16) == 0));
+  if (x8) {
+    const int half = a.rot / 2;
+    const long items = (long)n_rows * ((long)(nh + nkv) * (half / 8 + (hd - 2 * half) / 8) + (long)nkv * (vd / 8));
+    if (items < (1L << 31)) {
+      qkv_prepare_bf16x8_kernel<<<ceil_div(items, 256), 256, 0, stream>>>((bf16*)rows, (bf16*)kpages, (bf16*)vpages, (bf16*)keep, a, n_rows);
+      GIBBS_LAUNCH_STATUS("qkv_prepare");
+    }
+  }
   const int per_block = 4;
   const dim3 grid(n_rows, ceil_div(nh + 2 * nkv, per_block));
   if (dtype == GIBBS_F32)
