@@ -17,7 +17,7 @@
 // that are not 16-byte aligned; on the matrix cores for aligned bfloat16, float32 accumulators, the activation in
 // float32: tiles of 16 pairs for steps of few pairs (the experts' matrices are streamed once, a workgroup's four
 // waves split k, operands straight from memory: rows of h and of every W are contiguous along k), tiles of 128
-// pairs beyond (128 x 128 x 64 through LDS, double-buffered, as the framework's tiled product).
+// pairs beyond (128 pairs x 128 or 256 rows of W through LDS in tiles of 32 along k, double-buffered).
 #include "common.h"
 #include "activation.h"
 #include <algorithm>
@@ -242,8 +242,8 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 // Few pairs: a tile is 16 places, a workgroup takes 32 features of it (of both matrices, GLU) and its four waves a
 // quarter of k each, so that the experts' matrices, which are read once, are spread over many workgroups; the waves'
 // sums meet in LDS and the first wave adds them in wave order.  W is the first operand of the 16 x 16 x 32 product (the
-// tile is Y^T = W X^T): lane l holds the 8 values k = (l / 16) * 8 .. + 8 of feature or place l % 16, and its four
-// results are four neighbouring features of place l % 16.  Operands come straight from memory.
+// tile is Y^T = W X^T): lane l holds 8 values along k of feature or place l % 16, and its four results are four
+// neighbouring features of place l % 16.  Operands come straight from memory.
 template <bool GLU>
 __global__ __launch_bounds__(256) void moe_gemm_few_kernel(const bf16* __restrict__ X, long ldx, int top, const int* __restrict__ sorted_pair,
                                                            const int* __restrict__ tile_expert, const bf16* __restrict__ Wa,
@@ -265,21 +265,31 @@ __global__ __launch_bounds__(256) void moe_gemm_few_kernel(const bf16* __restric
   floatx4 acc[NA];
 #pragma unroll
   for (int t = 0; t < NA; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-  // wave w takes the steps of 32 along k whose number is w modulo 4
-  for (int k0 = wave * 32; k0 < I; k0 += 128) {
-    const int k = k0 + lg * 8;
-    const bf16x8 x8 = (src >= 0 && k < I) ? *(const bf16x8*)(xr + k) : zero8;
+  // wave w takes the stretches of 64 along k whose number is w modulo 4, in ascending order.  A lane group holds 16
+  // neighbouring values of a stretch as the operands of two products (the order along k inside a product is free as long as
+  // both operands agree), so that the wave asks for whole lines of 128 bytes of every row; two stretches at a time
+#pragma unroll 2
+  for (int k0 = wave * 64; k0 < I; k0 += 256) {
+    bf16x8 x8[2], a8[2][NF], b8[2][NF];
 #pragma unroll
-    for (int t = 0; t < NF; ++t) {
-      const int col = col0 + t * 16 + lr;
-      const bool in = col < O && k < I;
-      const bf16x8 a8 = in ? *(const bf16x8*)(wa + (size_t)col * I + k) : zero8;
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a8, x8, acc[t], 0, 0, 0);
-      if (GLU) {
-        const bf16x8 b8 = in ? *(const bf16x8*)(wb + (size_t)col * I + k) : zero8;
-        acc[NF + t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b8, x8, acc[NF + t], 0, 0, 0);
+    for (int u = 0; u < 2; ++u) {
+      const int k = k0 + lg * 16 + u * 8;
+      x8[u] = (src >= 0 && k < I) ? *(const bf16x8*)(xr + k) : zero8;
+#pragma unroll
+      for (int t = 0; t < NF; ++t) {
+        const int col = col0 + t * 16 + lr;
+        const bool in = col < O && k < I;
+        a8[u][t] = in ? *(const bf16x8*)(wa + (size_t)col * I + k) : zero8;
+        if (GLU) b8[u][t] = in ? *(const bf16x8*)(wb + (size_t)col * I + k) : zero8;
       }
     }
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int t = 0; t < NF; ++t) {
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a8[u][t], x8[u], acc[t], 0, 0, 0);
+        if (GLU) acc[NF + t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b8[u][t], x8[u], acc[NF + t], 0, 0, 0);
+      }
   }
 #pragma unroll
   for (int t = 0; t < NA; ++t)
@@ -303,27 +313,34 @@ __global__ __launch_bounds__(256) void moe_gemm_few_kernel(const bf16* __restric
     }
 }
 
-// Many pairs: a tile is 128 places, a workgroup of 4 waves computes 128 places x 128 features (GLU: 64 features of both
-// matrices), each wave 64 x 64 as 2 x 2 products of 32 x 32 x 16; tiles of 64 along k go through LDS (rows padded by 16
-// bytes against bank conflicts), double-buffered so that the next tile's loads are in flight while the matrix cores
-// work on the current one.  The rows of X are gathered by the tile's pairs as they are loaded.
-constexpr int TBM = 128, TBN = 128, TBK = 64, TLD = TBK + 8;
+// Many pairs: a tile is 128 places, a workgroup of NW waves computes 128 places x BN rows of W (GLU: BN / 2 features of both
+// matrices), each wave 64 x 64 as 2 x 2 products of 32 x 32 x 16; tiles of BK along k go through LDS (rows padded by 16
+// bytes against bank conflicts), double-buffered, and a further tile waits in registers, so that a tile's loads have
+// two tiles' work to arrive.  The rows of X are gathered by the tile's pairs as they are loaded.
+constexpr int TBM = 128;
+template <int BK, int BN>
 struct MoeTile {
-  bf16 a[TBM][TLD];
-  bf16 w[TBN][TLD];
+  bf16 a[TBM][BK + 8];
+  bf16 w[BN][BK + 8];
 };
-template <bool GLU>
-__global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(const bf16* __restrict__ X, long ldx, int top, const int* __restrict__ sorted_pair,
+template <bool GLU, int BK, int BN, int NW>
+__global__ __launch_bounds__(NW * WAVE) void moe_gemm_tiled_kernel(const bf16* __restrict__ X, long ldx, int top, const int* __restrict__ sorted_pair,
                                                              const int* __restrict__ tile_expert, const bf16* __restrict__ Wa,
                                                              const bf16* __restrict__ Wb, long expert_stride, bf16* __restrict__ Y, long ldy,
                                                              int O, int I, int act) {
+  using Tile = MoeTile<BK, BN>;
+  constexpr int KC = BK / 8;                        // chunks of 16 bytes in a row of a tile
+  constexpr int THREADS = NW * WAVE, WN = NW / 2;   // waves: 2 along the places, WN along the rows of W
+  constexpr int CA = TBM * KC / THREADS, CW = BN * KC / THREADS;   // chunks a thread moves per operand and tile of k
+  constexpr int NT = BN / WN / 32;                  // column blocks of 32 a wave
+  static_assert(CA >= 1 && CW >= 1 && NT >= (GLU ? 2 : 1) && NT % (GLU ? 2 : 1) == 0, "tile sizes");
   extern __shared__ __attribute__((aligned(16))) char moe_lds[];
-  MoeTile* tiles = (MoeTile*)moe_lds;               // [2]
-  int* srcs = (int*)(moe_lds + 2 * sizeof(MoeTile));   // [TBM]
+  Tile* tiles = (Tile*)moe_lds;                     // [2]
+  int* srcs = (int*)(moe_lds + 2 * sizeof(Tile));   // [TBM]
   const int tile = blockIdx.y, e = tile_expert[tile];
   if (e < 0) return;
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
-  constexpr int COLS = GLU ? TBN / 2 : TBN;         // features of the result that a workgroup takes
+  constexpr int COLS = GLU ? BN / 2 : BN;           // features of the result that a workgroup takes
   const int col0 = blockIdx.x * COLS;
   if (tid < TBM) {
     const int pair = sorted_pair[tile * TBM + tid];
@@ -332,68 +349,82 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(const bf16* __restr
   __syncthreads();
   const bf16* wa = Wa + (size_t)e * expert_stride;
   const bf16* wb = GLU ? Wb + (size_t)e * expert_stride : nullptr;
-  const int wr = (wave / 2) * 64;
-  // each thread moves 4 chunks of 16 bytes per operand and tile of k; its rows stay the same from tile to tile
-  const bf16* pa[4];
-  const bf16* pw[4];
+  const int wr = (wave / WN) * 64;
+  // a thread's rows stay the same from tile to tile
+  const bf16* pa[CA];
+  const bf16* pw[CW];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = (tid + i * 256) / 8;
+  for (int i = 0; i < CA; ++i) {
+    const int r = (tid + i * THREADS) / KC;
     pa[i] = srcs[r] >= 0 ? X + (size_t)srcs[r] * ldx : nullptr;
+  }
+#pragma unroll
+  for (int i = 0; i < CW; ++i) {
+    const int r = (tid + i * THREADS) / KC;
     const int col = col0 + (GLU ? r % COLS : r);
     pw[i] = col < O ? ((GLU && r >= COLS) ? wb : wa) + (size_t)col * I : nullptr;
   }
-  uint4 ra[4], rw[4];
-  auto load_global = [&](int k0) {
+  // two register sets take turns: a tile's loads are asked for two tiles ahead of its use
+  uint4 ra[2][CA], rw[2][CW];
+  auto load_global = [&](int k0, uint4* a, uint4* w) {
+    const int gk = k0 + (tid % KC) * 8;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int gk = k0 + ((tid + i * 256) % 8) * 8;
-      ra[i] = (pa[i] && gk < I) ? *(const uint4*)(pa[i] + gk) : make_uint4(0, 0, 0, 0);
-      rw[i] = (pw[i] && gk < I) ? *(const uint4*)(pw[i] + gk) : make_uint4(0, 0, 0, 0);
-    }
-  };
-  auto store_lds = [&](MoeTile& t) {
+    for (int i = 0; i < CA; ++i) a[i] = (pa[i] && gk < I) ? *(const uint4*)(pa[i] + gk) : make_uint4(0, 0, 0, 0);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = tid + i * 256, r = c / 8, kc = (c % 8) * 8;
-      *(uint4*)&t.a[r][kc] = ra[i];
-      *(uint4*)&t.w[r][kc] = rw[i];
-    }
+    for (int i = 0; i < CW; ++i) w[i] = (pw[i] && gk < I) ? *(const uint4*)(pw[i] + gk) : make_uint4(0, 0, 0, 0);
   };
-  floatx16 acc[2][2];
+  auto store_lds = [&](Tile& t, const uint4* a, const uint4* w) {
+    const int kc = (tid % KC) * 8;
+#pragma unroll
+    for (int i = 0; i < CA; ++i) *(uint4*)&t.a[(tid + i * THREADS) / KC][kc] = a[i];
+#pragma unroll
+    for (int i = 0; i < CW; ++i) *(uint4*)&t.w[(tid + i * THREADS) / KC][kc] = w[i];
+  };
+  floatx16 acc[2][NT];
 #pragma unroll
   for (int m = 0; m < 2; ++m)
 #pragma unroll
-    for (int n = 0; n < 2; ++n)
+    for (int n = 0; n < NT; ++n)
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[m][n][i] = 0.f;
-  // the wave's two column blocks of 32 in the W tile: neighbours (one matrix), or the same features of gate and up
-  const int wc0 = GLU ? (wave % 2) * 32 : (wave % 2) * 64;
-  const int wc1 = GLU ? COLS + wc0 : wc0 + 32;
-  const int n_tiles = (I + TBK - 1) / TBK;
-  load_global(0);
-  store_lds(tiles[0]);
-  __syncthreads();
-  for (int t = 0; t < n_tiles; ++t) {
-    const MoeTile& cur = tiles[t & 1];
-    if (t + 1 < n_tiles) load_global((t + 1) * TBK);
+  // the wave's column blocks of 32 in the W tile: neighbours (one matrix), or the same features of gate (the first half of
+  // its blocks) and up (the second half)
+  int wc[NT];
 #pragma unroll
-    for (int kk = 0; kk < TBK / 16; ++kk) {
-      bf16x8 fa[2], fw[2];
+  for (int n = 0; n < NT; ++n)
+    wc[n] = GLU ? (n / (NT / 2)) * COLS + (wave % WN) * (COLS / WN) + (n % (NT / 2)) * 32 : (wave % WN) * (BN / WN) + n * 32;
+  const int n_tiles = (I + BK - 1) / BK;
+  auto compute = [&](const Tile& cur) {
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      bf16x8 fa[2], fw[NT];
       const int k = kk * 16 + (lane / 32) * 8;
 #pragma unroll
       for (int m = 0; m < 2; ++m) fa[m] = *(const bf16x8*)&cur.a[wr + m * 32 + lane % 32][k];
-      fw[0] = *(const bf16x8*)&cur.w[wc0 + lane % 32][k];
-      fw[1] = *(const bf16x8*)&cur.w[wc1 + lane % 32][k];
+#pragma unroll
+      for (int n = 0; n < NT; ++n) fw[n] = *(const bf16x8*)&cur.w[wc[n] + lane % 32][k];
 #pragma unroll
       for (int m = 0; m < 2; ++m)
 #pragma unroll
-        for (int n = 0; n < 2; ++n) acc[m][n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[m], fw[n], acc[m][n], 0, 0, 0);
+        for (int n = 0; n < NT; ++n) acc[m][n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[m], fw[n], acc[m][n], 0, 0, 0);
     }
-    if (t + 1 < n_tiles) {
-      store_lds(tiles[(t + 1) & 1]);   // the other buffer: nobody reads it during this iteration
-      __syncthreads();
-    }
+  };
+  load_global(0, ra[0], rw[0]);
+  store_lds(tiles[0], ra[0], rw[0]);
+  load_global(BK, ra[0], rw[0]);
+  __syncthreads();
+  // tile t is in LDS buffer t % 2; while it is worked on, tile t + 1 waits in one register set and tile t + 2 is on its
+  // way into the other; a buffer is written again only after the barrier behind its last reader
+  // (an odd number of tiles is worked on as the next even one: loads beyond the inner size give zeros)
+  for (int t = 0; t < n_tiles; t += 2) {
+    load_global((t + 2) * BK, ra[1], rw[1]);
+    compute(tiles[0]);
+    store_lds(tiles[1], ra[0], rw[0]);
+    __syncthreads();
+    load_global((t + 3) * BK, ra[0], rw[0]);
+    compute(tiles[1]);
+    store_lds(tiles[0], ra[1], rw[1]);
+    __syncthreads();
   }
   // a lane holds column lane % 32 of a block and its rows (i / 4) * 8 + (lane / 32) * 4 + i % 4
 #pragma unroll
@@ -404,31 +435,43 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(const bf16* __restr
       if (srcs[row] < 0) continue;
       bf16* y = Y + (size_t)(tile * TBM + row) * ldy;
       if (GLU) {
-        const int col = col0 + wc0 + lane % 32;
-        if (col < O) y[col] = (bf16)(activate(acc[m][0][i], act) * acc[m][1][i]);
+#pragma unroll
+        for (int n = 0; n < NT / 2; ++n) {
+          const int col = col0 + wc[n] + lane % 32;
+          if (col < O) y[col] = (bf16)(activate(acc[m][n][i], act) * acc[m][NT / 2 + n][i]);
+        }
       } else {
 #pragma unroll
-        for (int n = 0; n < 2; ++n) {
-          const int col = col0 + wc0 + n * 32 + lane % 32;
+        for (int n = 0; n < NT; ++n) {
+          const int col = col0 + wc[n] + lane % 32;
           if (col < O) y[col] = (bf16)acc[m][n][i];
         }
       }
     }
 }
-constexpr int MOE_TILED_LDS = 2 * (int)sizeof(MoeTile) + TBM * (int)sizeof(int);
 
-template <bool GLU>
-int launch_tiled(const bf16* X, long ldx, int top, const int* sorted_pair, const int* tile_expert, int tiles, const bf16* wa, const bf16* wb,
-                 long stride, bf16* Y, long ldy, int O, int I, int act, hipStream_t stream) {
+template <bool GLU, int BK, int BN, int NW>
+int launch_tiled_as(const bf16* X, long ldx, int top, const int* sorted_pair, const int* tile_expert, int tiles, const bf16* wa, const bf16* wb,
+                    long stride, bf16* Y, long ldy, int O, int I, int act, hipStream_t stream) {
+  constexpr int LDS = 2 * (int)sizeof(MoeTile<BK, BN>) + TBM * (int)sizeof(int);
   static bool prepared = false;    // (one flag per instantiation)
   if (!prepared) {
-    hipError_t e = hipFuncSetAttribute((const void*)moe_gemm_tiled_kernel<GLU>, hipFuncAttributeMaxDynamicSharedMemorySize, MOE_TILED_LDS);
+    hipError_t e = hipFuncSetAttribute((const void*)moe_gemm_tiled_kernel<GLU, BK, BN, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
     if (e != hipSuccess) return gibbs_fail("moe_gemm: %s", hipGetErrorString(e));
     prepared = true;
   }
-  moe_gemm_tiled_kernel<GLU><<<dim3(ceil_div(O, GLU ? TBN / 2 : TBN), tiles), 256, MOE_TILED_LDS, stream>>>(X, ldx, top, sorted_pair, tile_expert, wa, wb,
-                                                                                                            stride, Y, ldy, O, I, act);
+  moe_gemm_tiled_kernel<GLU, BK, BN, NW><<<dim3(ceil_div(O, GLU ? BN / 2 : BN), tiles), NW * WAVE, LDS, stream>>>(X, ldx, top, sorted_pair, tile_expert, wa, wb,
+                                                                                                        stride, Y, ldy, O, I, act);
   return 0;
+}
+template <bool GLU>
+int launch_tiled(const bf16* X, long ldx, int top, const int* sorted_pair, const int* tile_expert, int tiles, const bf16* wa, const bf16* wb,
+                 long stride, bf16* Y, long ldy, int O, int I, int act, hipStream_t stream) {
+  // wide results with a long inner size: 256 rows of W a workgroup and 8 waves (the tile of X is read by half as many
+  // workgroups); otherwise 128 rows and 4 waves, which leaves more workgroups to spread
+  if (I > 1024 && O >= 512)
+    return launch_tiled_as<GLU, 32, 256, 8>(X, ldx, top, sorted_pair, tile_expert, tiles, wa, wb, stride, Y, ldy, O, I, act, stream);
+  return launch_tiled_as<GLU, 32, 128, 4>(X, ldx, top, sorted_pair, tile_expert, tiles, wa, wb, stride, Y, ldy, O, I, act, stream);
 }
 
 // ------------------------------------------------------------------------------------------------- combine
