@@ -62,6 +62,9 @@ int gibbs_gemm_heads_gated(const void* X, long ldx, long head_x, const void* W, 
 int gibbs_qk_unit_kv(void* rows, long ld, void* kpages, void* vpages, int dtype, const int* pos, const int* row_req,
                      const int* table, int max_pages, int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, int vd,
                      float eps, int unit, int norm_dim, float temp_coef, int temp_every, hipStream_t stream);
+int gibbs_rmsnorm_rows_mix_add_norm(float* x, const void* in, const int* place, const float* weight, int top, const void* shared,
+                                    const float* gate, const float* gain_d, float eps_d, const float* gain_n, float eps_n, void* out,
+                                    int dtype, int n, int hidden, hipStream_t stream);
 int gibbs_qkv_prepare(void* rows, long ld, void* kpages, void* vpages, int dtype, const float* bias, const float* inv_freq,
                       int rot, int variant, const float* cs_table, int table_len, void* keep, int keep_mode, int vt,
                       const float* lambda, const int* pos, const int* row_req, const int* table, int max_pages, int page_size,

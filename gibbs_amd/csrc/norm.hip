@@ -256,10 +256,20 @@ __global__ void rmsnorm_rows_add_kernel(float* __restrict__ x, const void* __res
 // part's result (one, in the activation type, or several in float32); and, with `out`, out = x * rsqrt(mean(x^2) + eps_n) *
 // gain_n of the new x (the next sublayer's norm).  A thread keeps its elements of the row in registers between the sums and
 // the scalings: 16-byte accesses, hidden sizes in steps of 4 up to 4 * CHUNKS * blockDim.  Sums, roots and x are float32.
-template <typename T, int CHUNKS>
+// MIX: the part's result is itself a weighted sum that no kernel has written yet (a mixture of experts' combination):
+// v = sum_s weight[n][s] * in[place[n][s]] (ascending s, rows of `in` in the activation type) + gate[n] * shared[n]
+// (shared null: none; gate null: 1), float32 throughout.
+struct RowMix {
+  const int* place;       // [n, top]
+  const float* weight;    // [n, top]
+  const void* shared;     // [n, hidden] or null
+  const float* gate;      // [n] or null
+  int top;
+};
+template <typename T, int CHUNKS, bool MIX>
 __global__ void rows_add_norm_vec_kernel(float* __restrict__ x, const void* __restrict__ in, int parts, size_t part_stride,
                                          const float* __restrict__ gain_d, float eps_d, const float* __restrict__ gain_n, float eps_n,
-                                         T* __restrict__ out, int hidden) {
+                                         T* __restrict__ out, int hidden, RowMix mix) {
   __shared__ float scratch[16];
   const size_t at = (size_t)blockIdx.x * hidden;
   float4 v[CHUNKS], xv[CHUNKS];
@@ -270,7 +280,19 @@ __global__ void rows_add_norm_vec_kernel(float* __restrict__ x, const void* __re
     v[c] = make_float4(0.f, 0.f, 0.f, 0.f);
     if (i < hidden) {
       xv[c] = *(const float4*)(x + at + i);
-      if (parts == 1) {
+      if (MIX) {
+        const size_t first = (size_t)blockIdx.x * mix.top;
+        for (int s = 0; s < mix.top; ++s) {
+          const float w = mix.weight[first + s];
+          const float4 r = load4((const T*)in + (size_t)mix.place[first + s] * hidden + i);
+          v[c].x = fmaf(w, r.x, v[c].x); v[c].y = fmaf(w, r.y, v[c].y); v[c].z = fmaf(w, r.z, v[c].z); v[c].w = fmaf(w, r.w, v[c].w);
+        }
+        if (mix.shared) {
+          const float g = mix.gate ? mix.gate[blockIdx.x] : 1.0f;
+          const float4 r = load4((const T*)mix.shared + at + i);
+          v[c].x = fmaf(g, r.x, v[c].x); v[c].y = fmaf(g, r.y, v[c].y); v[c].z = fmaf(g, r.z, v[c].z); v[c].w = fmaf(g, r.w, v[c].w);
+        }
+      } else if (parts == 1) {
         v[c] = load4((const T*)in + at + i);
       } else {
         for (int s = 0; s < parts; ++s) {
@@ -311,15 +333,20 @@ __global__ void rows_add_norm_vec_kernel(float* __restrict__ x, const void* __re
 
 template <typename T>
 bool launch_rows_add_norm(float* x, const void* in, int parts, long part_stride, const float* gain_d, float eps_d, const float* gain_n,
-                          float eps_n, T* out, int n, int hidden, hipStream_t stream) {
+                          float eps_n, T* out, int n, int hidden, hipStream_t stream, const RowMix* mixed = nullptr) {
   const uintptr_t vec = parts == 1 ? 4 * sizeof(T) : 16;
   if (hidden % 4 || ((uintptr_t)x % 16) || ((uintptr_t)in % vec) || (parts > 1 && part_stride % 4) || (gain_d && ((uintptr_t)gain_d % 16)) ||
-      (gain_n && ((uintptr_t)gain_n % 16)) || (out && ((uintptr_t)out % (4 * sizeof(T)))))
+      (gain_n && ((uintptr_t)gain_n % 16)) || (out && ((uintptr_t)out % (4 * sizeof(T)))) ||
+      (mixed && (parts != 1 || ((uintptr_t)mixed->shared % (4 * sizeof(T))))))
     return false;
   // (few rows: wide workgroups, every load of the row in flight at once)
   const int threads = hidden >= 4096 ? 1024 : (hidden >= 2048 ? 512 : (hidden >= 512 ? 256 : 64));
   const int chunks = ceil_div(hidden, 4 * threads);
-#define GIBBS_ROWS_ADD_NORM(C) rows_add_norm_vec_kernel<T, C><<<n, threads, 0, stream>>>(x, in, parts, (size_t)part_stride, gain_d, eps_d, gain_n, eps_n, out, hidden)
+#define GIBBS_ROWS_ADD_NORM(C)                                                                                                              \
+  do {                                                                                                                                      \
+    if (mixed) rows_add_norm_vec_kernel<T, C, true><<<n, threads, 0, stream>>>(x, in, parts, (size_t)part_stride, gain_d, eps_d, gain_n, eps_n, out, hidden, *mixed); \
+    else rows_add_norm_vec_kernel<T, C, false><<<n, threads, 0, stream>>>(x, in, parts, (size_t)part_stride, gain_d, eps_d, gain_n, eps_n, out, hidden, RowMix{}); \
+  } while (0)
   if (chunks == 1) GIBBS_ROWS_ADD_NORM(1);
   else if (chunks == 2) GIBBS_ROWS_ADD_NORM(2);
   else if (chunks <= 4) GIBBS_ROWS_ADD_NORM(4);
@@ -340,6 +367,22 @@ GIBBS_EXPORT int gibbs_rmsnorm_rows_add_norm(float* x, const void* in, int parts
   else return gibbs_fail("rmsnorm_rows_add_norm: unknown dtype %d", dtype);
   if (!queued) return -1;
   GIBBS_LAUNCH_STATUS("rmsnorm_rows_add_norm");
+}
+
+// The same with the part's result still to be summed: in [places, hidden] holds the results of a row's `top` choices at
+// place[n][s], v = sum_s weight[n][s] in[place[n][s]] + gate[n] shared[n] (a mixture of experts' combination, float32).
+GIBBS_EXPORT int gibbs_rmsnorm_rows_mix_add_norm(float* x, const void* in, const int* place, const float* weight, int top, const void* shared,
+                                                 const float* gate, const float* gain_d, float eps_d, const float* gain_n, float eps_n,
+                                                 void* out, int dtype, int n, int hidden, hipStream_t stream) {
+  GIBBS_REQUIRE(x && in && place && weight && out && n >= 0 && hidden > 0 && top >= 1, "rmsnorm_rows_mix_add_norm: bad sizes n=%d hidden=%d top=%d", n, hidden, top);
+  if (n == 0) return 0;
+  const RowMix mixed{place, weight, shared, gate, top};
+  bool queued;
+  if (dtype == GIBBS_F32) queued = launch_rows_add_norm<float>(x, in, 1, 0, gain_d, eps_d, gain_n, eps_n, (float*)out, n, hidden, stream, &mixed);
+  else if (dtype == GIBBS_BF16) queued = launch_rows_add_norm<bf16>(x, in, 1, 0, gain_d, eps_d, gain_n, eps_n, (bf16*)out, n, hidden, stream, &mixed);
+  else return gibbs_fail("rmsnorm_rows_mix_add_norm: unknown dtype %d", dtype);
+  if (!queued) return -1;
+  GIBBS_LAUNCH_STATUS("rmsnorm_rows_mix_add_norm");
 }
 
 GIBBS_EXPORT int gibbs_rmsnorm_rows_add(float* x, const void* in, int parts, long part_stride, const float* gain, float eps, int dtype,

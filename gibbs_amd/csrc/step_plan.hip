@@ -223,6 +223,26 @@ struct Exec {
   // rows that a body of this step has published for later bodies (an attention's values, for layers that mix them
   // into their own), by key; given back when the step ends
   std::map<int, void*> published;
+  // A mixture of experts' weighted sum that has not been written yet: the operation that adds the delta into the stream may
+  // sum it on its way (one kernel less, and the sum stays float32); whatever else comes first writes it (`mix_now`).
+  struct DeferredMix {
+    void* delta = nullptr;      // where the sum goes (null: nothing is deferred)
+    void* y = nullptr;          // [places, hidden]: the choices' results
+    int* place = nullptr;       // [n, top]
+    float* weight = nullptr;    // [n, top]
+    void* shared = nullptr;     // [n, hidden] or null
+    float* gate = nullptr;      // [n] or null
+    int top = 0;
+  } deferred;
+  void mix_done() {
+    give(deferred.shared);
+    give(deferred.y);
+    give(deferred.place);
+    give(deferred.weight);
+    give(deferred.gate);
+    deferred = DeferredMix{};
+  }
+  void mix_now();
   Exec(const Plan& plan, const GibbsStepArgs& args);
   void* take(long bytes) {
     void* ptr = arena.take(bytes);
@@ -983,12 +1003,10 @@ struct MoeBody : Body {
       e.give(sy);
     }
     Pending delta{e.take((long)N * W * e.esize), 1};
-    RUN(e, gibbs_moe_combine(y, place, weight, shared, sgate, delta.data, e.p.dtype, N, top, W, e.a.stream));
-    e.give(shared);
-    e.give(y);
-    e.give(place);
-    e.give(weight);
-    e.give(sgate);
+    e.mix_now();      // (an earlier sum that nothing has taken yet)
+    e.deferred.delta = delta.data;
+    e.deferred.y = y; e.deferred.place = place; e.deferred.weight = weight; e.deferred.shared = shared; e.deferred.gate = sgate;
+    e.deferred.top = top;
     return delta;
   }
 };
@@ -1009,6 +1027,13 @@ struct HostBody : Body {
 };
 
 // ------------------------------------------------------------------------------------------------- the step
+void Exec::mix_now() {
+  if (!deferred.delta) return;
+  RUN(*this, gibbs_moe_combine(deferred.y, deferred.place, deferred.weight, deferred.shared, deferred.gate, deferred.delta, p.dtype, a.n_rows,
+                               deferred.top, p.hidden, a.stream));
+  mix_done();
+}
+
 void Exec::run() {
   const int N = a.n_rows, H = p.hidden;
   float* x = a.x_in;
@@ -1037,6 +1062,7 @@ void Exec::run() {
   const int first = whole ? 0 : a.first_op, last = whole ? (int)p.ops.size() : a.first_op + a.n_ops;
   for (int i = first; i < last && ok(); ++i) {
     const Plan::Op& op = p.ops[i];
+    if (deferred.delta && op.kind != Plan::OP_ADD_NORMED && !(op.kind == Plan::OP_DROP && deltas[op.value].data != deferred.delta)) mix_now();
     switch (op.kind) {
       case Plan::OP_HALF: {
         const NormPart& n = *p.norms[op.norm];
@@ -1082,12 +1108,16 @@ void Exec::run() {
         if (next && pending.parts == 0 && d.data && p.norms[op.norm]->plain_rms(&gain_d, &eps_d) && p.norms[next->norm]->plain_rms(&gain_n, &eps_n)) {
           void* out = take((long)N * H * esize);
           int fused = -1;
+          const bool mixed = deferred.delta && deferred.delta == d.data;
           if (!dry && status == 0) {
-            fused = gibbs_rmsnorm_rows_add_norm(x, d.data, std::max(d.parts, 1), (long)N * H, gain_d, eps_d, gain_n, eps_n, out, p.dtype, N, H, a.stream);
+            fused = mixed ? gibbs_rmsnorm_rows_mix_add_norm(x, deferred.y, deferred.place, deferred.weight, deferred.top, deferred.shared, deferred.gate,
+                                                            gain_d, eps_d, gain_n, eps_n, out, p.dtype, N, H, a.stream)
+                          : gibbs_rmsnorm_rows_add_norm(x, d.data, std::max(d.parts, 1), (long)N * H, gain_d, eps_d, gain_n, eps_n, out, p.dtype, N, H, a.stream);
             if (fused > 0) status = 1;
           } else if (H % 4 == 0 && H <= 16384) {
             fused = 0;      // (a dry run: the same buffers as the real one will take)
           }
+          if (fused == 0 && mixed) mix_done();
           if (fused == 0) {
             give(d.data);
             d = Pending{};
@@ -1099,6 +1129,7 @@ void Exec::run() {
           }
           give(out);
         }
+        mix_now();
         // (what is pending stays pending: additions into x commute, and the next norm still takes it on its way)
         if (p.norms[op.norm]->add_normed(*this, x, deltas[op.value])) {
           deltas[op.value] = Pending{};
@@ -1151,6 +1182,7 @@ void Exec::run() {
         break;
     }
   }
+  mix_now();
   if (whole && a.n_logits > 0 && ok()) {
     // (several streams: the model's output is their sum)
     void* h = S > 1 ? p.norms[p.tail]->run_streams(*this, x, S, nullptr, a.logit_rows, a.n_logits)
@@ -1610,6 +1642,7 @@ GIBBS_EXPORT long gibbs_plan_body_forward(const void* plan, int body, const Gibb
   if (g >= 0 && !(g < args->n_groups && args->tables && args->tables[g] && args->widths[g] > 0)) return gibbs_fail("body: no block table for cache group %d", g), -1;
   Exec e(*p, *args);
   Pending delta = p->bodies[body]->general(e, (void*)h);
+  e.mix_now();
   if (e.status) return -1;
   if (e.dry) return e.arena.peak;
   *out_offset = (char*)delta.data - (char*)args->workspace;
