@@ -39,32 +39,67 @@ __device__ __forceinline__ void store4f(bf16* p, float4 v) {
   o.h[0] = (bf16)v.x; o.h[1] = (bf16)v.y; o.h[2] = (bf16)v.z; o.h[3] = (bf16)v.w;
   *(uint2*)p = o.u;
 }
-// One wave's inner product of a row with a float32 vector; `vec`: the width is a multiple of 4 and both are aligned, so a
-// lane takes 4 neighbouring values at a time (the order of the additions depends on the width alone).
-template <typename T>
-__device__ __forceinline__ float wave_dot(const T* __restrict__ row, const float* __restrict__ w, int W, int lane, bool vec) {
-  float s = 0.f;
+// One wave's inner products of a row with NV float32 vectors (the row is loaded once); `vec`: the width is a multiple of 4
+// and all are aligned, so a lane takes 4 neighbouring values at a time.  Every sum is one chain of additions in ascending
+// k per lane, so its value depends on the width alone, not on NV or on how many steps are asked for together.
+template <typename T, int NV>
+__device__ __forceinline__ void wave_dots(const T* __restrict__ row, const float* const (&w)[NV], float (&out)[NV], int W, int lane, bool vec) {
+  float s[NV];
+#pragma unroll
+  for (int v = 0; v < NV; ++v) s[v] = 0.f;
   if (vec) {
-    // (four steps at a time: their loads are asked for together)
     int k = lane * 4;
+    // (eight steps at a time, then four: their loads are asked for together)
+    for (; k + 7 * WAVE * 4 < W; k += 8 * WAVE * 4) {
+      float4 a[8], b[NV][8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        a[u] = load4f(row + k + u * WAVE * 4);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) b[v][u] = *(const float4*)(w[v] + k + u * WAVE * 4);
+      }
+#pragma unroll
+      for (int v = 0; v < NV; ++v)
+#pragma unroll
+        for (int u = 0; u < 8; ++u) { s[v] = fmaf(a[u].x, b[v][u].x, s[v]); s[v] = fmaf(a[u].y, b[v][u].y, s[v]); s[v] = fmaf(a[u].z, b[v][u].z, s[v]); s[v] = fmaf(a[u].w, b[v][u].w, s[v]); }
+    }
     for (; k + 3 * WAVE * 4 < W; k += 4 * WAVE * 4) {
-      float4 a[4], b[4];
+      float4 a[4], b[NV][4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         a[u] = load4f(row + k + u * WAVE * 4);
-        b[u] = *(const float4*)(w + k + u * WAVE * 4);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) b[v][u] = *(const float4*)(w[v] + k + u * WAVE * 4);
       }
 #pragma unroll
-      for (int u = 0; u < 4; ++u) { s = fmaf(a[u].x, b[u].x, s); s = fmaf(a[u].y, b[u].y, s); s = fmaf(a[u].z, b[u].z, s); s = fmaf(a[u].w, b[u].w, s); }
+      for (int v = 0; v < NV; ++v)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) { s[v] = fmaf(a[u].x, b[v][u].x, s[v]); s[v] = fmaf(a[u].y, b[v][u].y, s[v]); s[v] = fmaf(a[u].z, b[v][u].z, s[v]); s[v] = fmaf(a[u].w, b[v][u].w, s[v]); }
     }
     for (; k < W; k += WAVE * 4) {
-      const float4 a = load4f(row + k), b = *(const float4*)(w + k);
-      s = fmaf(a.x, b.x, s); s = fmaf(a.y, b.y, s); s = fmaf(a.z, b.z, s); s = fmaf(a.w, b.w, s);
+      const float4 a = load4f(row + k);
+#pragma unroll
+      for (int v = 0; v < NV; ++v) {
+        const float4 c = *(const float4*)(w[v] + k);
+        s[v] = fmaf(a.x, c.x, s[v]); s[v] = fmaf(a.y, c.y, s[v]); s[v] = fmaf(a.z, c.z, s[v]); s[v] = fmaf(a.w, c.w, s[v]);
+      }
     }
   } else {
-    for (int k = lane; k < W; k += WAVE) s = fmaf(to_float(row[k]), w[k], s);
+    for (int k = lane; k < W; k += WAVE) {
+      const float a = to_float(row[k]);
+#pragma unroll
+      for (int v = 0; v < NV; ++v) s[v] = fmaf(a, w[v][k], s[v]);
+    }
   }
-  return wave_sum(s);
+#pragma unroll
+  for (int v = 0; v < NV; ++v) out[v] = wave_sum(s[v]);
+}
+template <typename T>
+__device__ __forceinline__ float wave_dot(const T* __restrict__ row, const float* __restrict__ w, int W, int lane, bool vec) {
+  const float* const ws[1] = {w};
+  float out[1];
+  wave_dots<T, 1>(row, ws, out, W, lane, vec);
+  return out[0];
 }
 
 template <typename T>
@@ -76,11 +111,23 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const T* __restrict__ h
   const int n = blockIdx.x, wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, n_waves = blockDim.x / WAVE;
   const T* row = h + (size_t)n * ldh;
   const bool vec = W % 4 == 0 && ldh % 4 == 0 && ((uintptr_t)h % 16) == 0 && ((uintptr_t)router % 16) == 0 && ((uintptr_t)shared_gate % 16) == 0;
+  // the last wave also has the shared expert's gate: with its last expert's logit in one pass over the row
+  bool gate_left = shared_gate && wave == n_waves - 1;
   for (int e = wave; e < E; e += n_waves) {
-    const float s = wave_dot(row, router + (size_t)e * W, W, lane, vec);
+    float s;
+    if (gate_left && e + n_waves >= E) {
+      const float* const ws[2] = {router + (size_t)e * W, shared_gate};
+      float both[2];
+      wave_dots<T, 2>(row, ws, both, W, lane, vec);
+      s = both[0];
+      if (lane == 0) sgate[n] = 1.0f / (1.0f + expf(-both[1]));
+      gate_left = false;
+    } else {
+      s = wave_dot(row, router + (size_t)e * W, W, lane, vec);
+    }
     if (lane == 0) z[e] = s + (router_bias ? router_bias[e] : 0.f);
   }
-  if (shared_gate && wave == n_waves - 1) {
+  if (gate_left) {
     const float s = wave_dot(row, shared_gate, W, lane, vec);
     if (lane == 0) sgate[n] = 1.0f / (1.0f + expf(-s));
   }
