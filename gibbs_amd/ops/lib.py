@@ -93,6 +93,8 @@ _SIGNATURES = {
     "gibbs_moe_gemm": [c_void_p, c_long, c_int, c_void_p, c_void_p, c_long, c_int, c_void_p, c_void_p, c_void_p, c_long, c_int, c_int,
                        c_int, c_int, c_void_p],
     "gibbs_moe_combine": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "gibbs_rmsnorm_rows_mix_add_norm": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_float, c_void_p,
+                                        c_float, c_void_p, c_int, c_int, c_int, c_void_p],
     "gibbs_causal_conv_silu": [c_void_p, c_long, c_int, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gibbs_delta_rule": [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p, c_long, c_void_p,

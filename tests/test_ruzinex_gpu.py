@@ -300,6 +300,7 @@ def test_grouped_heads_far_keys_page_borders_and_the_sink(kernel):
 
 
 @pytest.mark.parametrize("case", [(torch.float32, 52, 7, 3, 100, 30), (torch.bfloat16, 52, 7, 3, 100, 30), (torch.bfloat16, 300, 8, 2, 128, 64),
+                                  (torch.bfloat16, 300, 3, 2, 1056, 512),
                                   (torch.bfloat16, 9, 16, 4, 64, 32), (torch.float32, 3, 1, 1, 24, 8)])
 def test_experts_route_group_products_and_combine(case):
     """The router's choices and weights (with made-up logits that tie), the pairs sorted by expert, both products and the
@@ -362,6 +363,37 @@ def test_experts_route_group_products_and_combine(case):
             want[r] += wt[r, c] * ((Z.silu(hh[r] @ g64[e].T) * (hh[r] @ u64[e].T)) @ d64[e].T)
     tol = 2e-5 if dtype == torch.float32 else 3e-2
     assert np.abs(out.float().cpu().numpy() - want).max() <= tol * max(1.0, np.abs(want).max())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shared", ["gated", "plain", "none"])
+def test_experts_sum_inside_the_sublayer_boundary(dtype, shared):
+    """x += gain_b * rms_norm(sum_s w[n][s] y[place[n][s]] + g[n] shared[n]) and out = gain_a * rms_norm(x) in one kernel, against
+    numpy; places are scattered over more rows than are used, and one row's weights leave a single choice."""
+    from gibbs_amd.ops.lib import call, dtype_code, ptr, stream
+    rng = np.random.default_rng(11)
+    n, top, W, places = 37, 3, 200, 150
+    y = _dev(rng.normal(size=(places, W)), dtype)
+    place = rng.permutation(places)[:n * top].reshape(n, top).astype(np.int32)
+    weight = rng.random(size=(n, top)).astype(np.float32)
+    weight[5] = [0.0, 1.0, 0.0]
+    sh = _dev(rng.normal(size=(n, W)), dtype) if shared != "none" else None
+    g = _dev(rng.random(size=n)) if shared == "gated" else None
+    x0 = rng.normal(size=(n, W)).astype(np.float32)
+    gain_b, gain_a = rng.normal(size=W).astype(np.float32), rng.normal(size=W).astype(np.float32)
+    x = _dev(x0)
+    out = torch.empty((n, W), dtype=dtype, device="cuda")
+    gb, ga, pl, wt = _dev(gain_b), _dev(gain_a), torch.tensor(place, device="cuda"), _dev(weight)
+    call("gibbs_rmsnorm_rows_mix_add_norm", ptr(x), ptr(y), ptr(pl), ptr(wt), top, ptr(sh) if sh is not None else None,
+         ptr(g) if g is not None else None, ptr(gb), 1e-5, ptr(ga), 1e-6, ptr(out), dtype_code(dtype), n, W, stream())
+    y64 = y.float().cpu().numpy().astype(np.float64)
+    v = (weight.astype(np.float64)[:, :, None] * y64[place]).sum(1)
+    if sh is not None:
+        v += (g.cpu().numpy().astype(np.float64)[:, None] if g is not None else 1.0) * sh.float().cpu().numpy().astype(np.float64)
+    want_x = x0 + Z.rms_norm(v, gain_b.astype(np.float64), 1e-5)
+    want_out = Z.rms_norm(want_x, gain_a.astype(np.float64), 1e-6)
+    assert np.abs(x.cpu().numpy() - want_x).max() <= 2e-5
+    assert np.abs(out.float().cpu().numpy() - want_out).max() <= (2e-5 if dtype == torch.float32 else 2e-2) * max(1.0, np.abs(want_out).max())
 
 
 def test_a_rows_experts_do_not_depend_on_its_neighbours():
