@@ -15,11 +15,13 @@ from typing import Any, Mapping, Optional, Sequence, Tuple, Union
 
 @dataclass(frozen=True)
 class NormSpec:
-    """A normalisation over the last axis. `kind` selects the part (`"rms"`; `"layer"`: mean taken off, gain and bias)."""
+    """A normalisation over the last axis. `kind` selects the part (`"rms"`; `"layer"`: mean taken off, gain and bias;
+    `"group_rms"`: the row in `groups` equal consecutive parts, each divided by its own root mean square)."""
     kind: str
     eps: float
     weight: str                     # tensor name of the gain
     bias: Optional[str] = None      # tensor name of the bias (kinds that have one)
+    groups: int = 1                 # parts of the row that are normed by themselves (kind "group_rms")
 
 
 @dataclass(frozen=True)
@@ -150,6 +152,8 @@ class ModelSpec:
     # residual streams (every stream starts as the embedding's output; the model's output is their sum).
     embedding_tables: Optional[EmbeddingTablesSpec] = None
     streams: int = 1
+    # logits <- cap * tanh(logits / cap) after the head (0: not capped)
+    logit_softcap: float = 0.0
     # (name, shape) of checkpoint tensors that belong to the model and that no part reads (a layer without a
     # feed-forward whose checkpoint holds that sublayer's norm all the same)
     unread_tensors: Tuple[Tuple[str, Tuple[int, ...]], ...] = ()

@@ -3,8 +3,9 @@
 // own absolute position and request.
 //
 //   row n, head h (kv head g = h / (nh / nkv)), position p = pos[n], request r = row_req[n]:
-//   visible keys are lo .. p with lo = max(0, p - window + 1) (window 0: all keys);
-//   s_k = (q . K[k]) * scale (+ slopes[h] * (k - p) when the position encoding is a linear bias over
+//   visible keys are lo .. p with lo = max(0, p - window + 1) (window 0: all keys), or with `chunk` > 0
+//   lo = p - p % chunk (the keys of the row's own stretch of `chunk` positions, counted from position 0);
+//   s_k = (q . K[k]) * scale, then with `softcap` > 0  s_k = softcap * tanh(s_k / softcap), then (+ slopes[h] * (k - p) when the position encoding is a linear bias over
 //   the distance; + bias[min(p - k, bias_len - 1)][h] when it is a table over the distance);
 //   out = sum_k softmax(s)_k V[k], maxima and sums in float32.  Values may have a head size of their
 //   own (vd): value pages are [page, kv head, slot in page, vd] and a row of out holds nh * vd.
@@ -33,6 +34,8 @@ struct AttnArgs {
   const float* bias;    // [bias_len, nh] or null: s_k += bias[min(p - k, bias_len - 1)][h]
   int bias_len;
   const float* sink;    // [nh] or null: the softmax's denominator also holds exp(sink[h]) (no key, no value, not scaled)
+  int chunk;            // > 0: a row sees the keys of its own stretch of `chunk` positions only
+  float softcap;        // > 0: scores are capped as softcap * tanh(s / softcap) before any bias
 };
 
 template <typename T>
@@ -55,7 +58,7 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(const T* __restric
   if (!active) return;
 
   const int hi = p;
-  const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
+  const int lo = a.chunk > 0 ? p - p % a.chunk : (a.window > 0 ? max(0, p - a.window + 1) : 0);
   float m = -INFINITY, l = 0.f;
   float acc[DPL] = {};
 
@@ -74,6 +77,7 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(const T* __restric
       float dot = 0.f;
       for (int e = 0; e < hd; ++e) dot = fmaf(sq[wave][e], to_float(kr[e]), dot);
       s = dot * a.scale;
+      if (a.softcap > 0.f) s = a.softcap * tanhf(s / a.softcap);
       if (a.slopes) s += a.slopes[h] * (float)(key - p);
       if (a.bias) s += a.bias[(size_t)min(p - key, a.bias_len - 1) * a.nh + h];
     }
@@ -108,19 +112,21 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(const T* __restric
 
 // The general entry point: values of head size vd, an optional table of score biases over the distance, and an
 // optional sink per head (a term exp(sink[h]) in the softmax's denominator that has no key and no value).
-GIBBS_EXPORT int gibbs_attention_plain_sink(const void* q, const void* kpages, const void* vpages, void* out, int dtype,
-                                            const int* pos, const int* row_req, const int* table, int max_pages,
-                                            int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, int vd,
-                                            long ldq, long ldo, float scale, int window, const float* slopes,
-                                            const float* bias, int bias_len, const float* sink, hipStream_t stream) {
+GIBBS_EXPORT int gibbs_attention_plain_masked(const void* q, const void* kpages, const void* vpages, void* out, int dtype,
+                                              const int* pos, const int* row_req, const int* table, int max_pages,
+                                              int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, int vd,
+                                              long ldq, long ldo, float scale, int window, const float* slopes,
+                                              const float* bias, int bias_len, const float* sink, int chunk, float softcap,
+                                              hipStream_t stream) {
   GIBBS_REQUIRE(n_rows >= 0 && nh > 0 && nkv > 0 && hd > 0 && vd > 0, "attention: bad sizes rows=%d heads=%d kv=%d hd=%d vd=%d", n_rows, nh, nkv, hd, vd);
   GIBBS_REQUIRE(nh % nkv == 0, "attention: %d heads are not a multiple of %d kv heads", nh, nkv);
   GIBBS_REQUIRE(hd <= MAX_HD && vd <= MAX_HD, "attention: head sizes %d, %d above %d", hd, vd, MAX_HD);
   GIBBS_REQUIRE(ldq >= (long)nh * hd && ldo >= (long)nh * vd, "attention: row strides shorter than heads * head size");
   GIBBS_REQUIRE(page_size > 0 && max_pages > 0 && num_pages > 0 && window >= 0, "attention: bad cache geometry");
   GIBBS_REQUIRE(!bias || bias_len > 0, "attention: an empty table of score biases");
+  GIBBS_REQUIRE(chunk >= 0 && !(chunk > 0 && window > 0) && softcap >= 0.f, "attention: a window of %d with chunks of %d, scores capped at %g", window, chunk, softcap);
   if (n_rows == 0) return 0;
-  AttnArgs a{pos, row_req, table, max_pages, page_size, num_pages, nh, nkv, hd, ldq, ldo, scale, window, slopes, vd, bias, bias_len, sink};
+  AttnArgs a{pos, row_req, table, max_pages, page_size, num_pages, nh, nkv, hd, ldq, ldo, scale, window, slopes, vd, bias, bias_len, sink, chunk, softcap};
   dim3 grid(n_rows, ceil_div(nh, 4));
   GIBBS_REQUIRE(grid.y <= 65535, "attention: too many heads (%d)", nh);
   if (dtype == GIBBS_F32)
@@ -130,6 +136,15 @@ GIBBS_EXPORT int gibbs_attention_plain_sink(const void* q, const void* kpages, c
   else
     return gibbs_fail("attention: unknown dtype %d", dtype);
   GIBBS_LAUNCH_STATUS("attention");
+}
+
+GIBBS_EXPORT int gibbs_attention_plain_sink(const void* q, const void* kpages, const void* vpages, void* out, int dtype,
+                                            const int* pos, const int* row_req, const int* table, int max_pages,
+                                            int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, int vd,
+                                            long ldq, long ldo, float scale, int window, const float* slopes,
+                                            const float* bias, int bias_len, const float* sink, hipStream_t stream) {
+  return gibbs_attention_plain_masked(q, kpages, vpages, out, dtype, pos, row_req, table, max_pages, page_size, num_pages, n_rows, nh,
+                                      nkv, hd, vd, ldq, ldo, scale, window, slopes, bias, bias_len, sink, 0, 0.f, stream);
 }
 
 GIBBS_EXPORT int gibbs_attention_plain_general(const void* q, const void* kpages, const void* vpages, void* out, int dtype,

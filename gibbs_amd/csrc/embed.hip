@@ -51,3 +51,15 @@ GIBBS_EXPORT int gibbs_embed(const void* table, int dtype, const int* ids, float
                              int hidden, int vocab, hipStream_t stream) {
   return gibbs_embed_general(table, dtype, ids, x, mirror, n, hidden, vocab, 1.0f, nullptr, nullptr, nullptr, stream);
 }
+
+// The model's other end: logits capped in place, v <- cap * tanh(v / cap) (float32).
+__global__ void softcap_kernel(float* __restrict__ v, long count, float cap) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) v[i] = cap * tanhf(v[i] / cap);
+}
+GIBBS_EXPORT int gibbs_softcap_rows(float* v, long count, float cap, hipStream_t stream) {
+  GIBBS_REQUIRE(v && count >= 0 && cap > 0.f, "softcap: bad operands count=%ld cap=%g", count, cap);
+  if (count == 0) return 0;
+  softcap_kernel<<<ceil_div(count, 256), 256, 0, stream>>>(v, count, cap);
+  GIBBS_LAUNCH_STATUS("softcap");
+}

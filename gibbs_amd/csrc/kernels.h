@@ -22,6 +22,10 @@ int gibbs_attention_plain_general(const void* q, const void* kpages, const void*
                                   const int* row_req, const int* table, int max_pages, int page_size, int num_pages, int n_rows,
                                   int nh, int nkv, int hd, int vd, long ldq, long ldo, float scale, int window,
                                   const float* slopes, const float* bias, int bias_len, hipStream_t stream);
+int gibbs_attention_plain_masked(const void* q, const void* kpages, const void* vpages, void* out, int dtype, const int* pos,
+                                 const int* row_req, const int* table, int max_pages, int page_size, int num_pages, int n_rows,
+                                 int nh, int nkv, int hd, int vd, long ldq, long ldo, float scale, int window, const float* slopes,
+                                 const float* bias, int bias_len, const float* sink, int chunk, float softcap, hipStream_t stream);
 int gibbs_attention_plain_sink(const void* q, const void* kpages, const void* vpages, void* out, int dtype, const int* pos,
                                const int* row_req, const int* table, int max_pages, int page_size, int num_pages, int n_rows,
                                int nh, int nkv, int hd, int vd, long ldq, long ldo, float scale, int window,
@@ -69,11 +73,22 @@ int gibbs_qkv_prepare(void* rows, long ld, void* kpages, void* vpages, int dtype
                       int rot, int variant, const float* cs_table, int table_len, void* keep, int keep_mode, int vt,
                       const float* lambda, const int* pos, const int* row_req, const int* table, int max_pages, int page_size,
                       int num_pages, int n_rows, int nh, int nkv, int hd, int vd, hipStream_t stream);
+int gibbs_qkv_prepare_full(void* rows, long ld, void* kpages, void* vpages, int dtype, const float* bias, const float* inv_freq,
+                           int rot, int variant, const float* cs_table, int table_len, void* keep, int keep_mode, int vt,
+                           const float* lambda, const int* pos, const int* row_req, const int* table, int max_pages, int page_size,
+                           int num_pages, int n_rows, int nh, int nkv, int hd, int vd, const float* q_gain, const float* k_gain,
+                           float qk_eps, int norm_dim, int v_from_k, const float* v_inv_freq, int v_rot, hipStream_t stream);
+int gibbs_attention_finish(void* att, long ldo, const void* gate, long ld_gate, int gate_head, int dtype, const int* pos,
+                           const float* v_inv_freq, int v_rot, int variant, int n_rows, int nh, int vd, int vt, hipStream_t stream);
 // ---- moe.hip: mixture of experts
 long gibbs_moe_capacity(int n_pairs, int E, int bm);
 int gibbs_moe_tile(int n_pairs, int E);
 int gibbs_moe_route(const void* h, long ldh, int dtype, const float* router, const float* router_bias, const float* shared_gate,
                     int* chosen, float* weight, float* sgate, int n, int W, int E, int top, hipStream_t stream);
+int gibbs_moe_route_mode(const void* h, long ldh, int dtype, const float* router, const float* router_bias, const float* shared_gate,
+                         int* chosen, float* weight, float* sgate, int n, int W, int E, int top, int mode, hipStream_t stream);
+int gibbs_moe_combine_self(const void* y, const int* pair_pos, const float* weight, const void* shared, const float* sgate,
+                           const void* self, void* out, int dtype, int n, int top, int W, hipStream_t stream);
 int gibbs_moe_group(const int* chosen, int n_pairs, int E, int bm, int* sorted_pair, int* pair_pos, int* tile_expert, long cap,
                     hipStream_t stream);
 int gibbs_moe_gemm(const void* X, long ldx, int top, const int* sorted_pair, const int* tile_expert, long cap, int bm,
@@ -83,6 +98,22 @@ int gibbs_moe_combine(const void* y, const int* pair_pos, const float* weight, c
 int gibbs_causal_conv_silu(const void* in, long ld, int dtype, const float* taps, float* state, long slot_stride,
                            const int* row_req, const int* cu, const int* slot, float* out, int n_rows, int n_req, int C, int K,
                            int update_state, int single_rows, hipStream_t stream);
+int gibbs_causal_conv(const void* in, long ld, int dtype, const float* taps, const float* bias, float* state, long slot_stride,
+                      const int* row_req, const int* cu, const int* slot, void* out, int out_f32, long ld_out, int n_rows, int n_req,
+                      int C, int K, int act, int residual, int update_state, int single_rows, hipStream_t stream);
+int gibbs_ssd_prep(const float* xbc, long ld_x, const void* dt_raw, long ld_raw, int dtype, const float* dt_bias, const float* a_log,
+                   float* decay, float* xdt, int n_rows, int H, int V, hipStream_t stream);
+int gibbs_ssd_rule(const float* q, const float* k, long ldqk, const float* v, long ldv, const float* decay, float* state,
+                   long slot_stride, const int* cu, const int* slot, float* out, int n_req, int H, int G, int D, int V,
+                   hipStream_t stream);
+int gibbs_softcap_rows(float* v, long count, float cap, hipStream_t stream);
+// ---- norm_groups.hip: RMS norm in groups
+int gibbs_group_rmsnorm(float* x, const void* delta, int parts, long part_stride, const float* gain_d, float eps_d, int groups_d,
+                        const float* gain_n, float eps_n, int groups_n, void* out, int dtype, const int* rows, int n_out, int H,
+                        hipStream_t stream);
+int gibbs_gated_group_norm(const float* in, const float* skip, long ld_skip, const float* skip_w, int skip_len, const void* gate,
+                           long ld_gate, const float* gain, float eps, int groups, void* y, int dtype, int n, int C,
+                           hipStream_t stream);
 int gibbs_delta_prep(float* q, float* k, long ldqk, const void* beta_raw, const void* a_head, long ld_raw, int dtype,
                      const float* a_channel, const float* dt_bias, const float* a_log, float* beta, float* decay, int n_rows,
                      int G, int H, int D, float q_scale, float unit_eps, hipStream_t stream);

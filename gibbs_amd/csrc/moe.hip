@@ -3,6 +3,9 @@
 //
 //   route      z = W_r h + b in float32 (h as the step holds it); the `top` largest logits (the lower index among
 //              equals); weights = softmax over the chosen logits alone; gate = sigmoid(w_sg . h) for the shared expert
+//              (mode 1: scores s = softmax(z) over all router outputs; the `top` largest of s + correction; weights = the
+//              chosen scores s divided by their sum + 1e-20.  Router outputs from `E_real` on are identity experts: they
+//              have no matrices, their result is the row itself, and their pairs take no place in the tiles)
 //   group      the step's (row, choice) pairs sorted by expert into tiles of `bm` pairs that belong to one expert
 //              each (every expert's stretch is padded to whole tiles); nothing goes back to the host, so a step
 //              with experts can be captured in a graph: the products below run over the worst-case number of tiles
@@ -106,8 +109,8 @@ template <typename T>
 __global__ __launch_bounds__(1024) void moe_route_kernel(const T* __restrict__ h, long ldh, const float* __restrict__ router,
                                                         const float* __restrict__ router_bias, const float* __restrict__ shared_gate,
                                                         int* __restrict__ chosen, float* __restrict__ weight, float* __restrict__ sgate,
-                                                        int W, int E, int top) {
-  extern __shared__ float z[];   // [E]
+                                                        int W, int E, int top, int mode) {
+  extern __shared__ float z[];   // [E] (mode 1: and the scores behind them, [E])
   const int n = blockIdx.x, wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, n_waves = blockDim.x / WAVE;
   const T* row = h + (size_t)n * ldh;
   const bool vec = W % 4 == 0 && ldh % 4 == 0 && ((uintptr_t)h % 16) == 0 && ((uintptr_t)router % 16) == 0 && ((uintptr_t)shared_gate % 16) == 0;
@@ -125,7 +128,7 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const T* __restrict__ h
     } else {
       s = wave_dot(row, router + (size_t)e * W, W, lane, vec);
     }
-    if (lane == 0) z[e] = s + (router_bias ? router_bias[e] : 0.f);
+    if (lane == 0) z[e] = s + ((router_bias && mode == 0) ? router_bias[e] : 0.f);
   }
   if (gate_left) {
     const float s = wave_dot(row, shared_gate, W, lane, vec);
@@ -138,6 +141,23 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const T* __restrict__ h
   // over the chosen logits alone
   int* mine = chosen + (size_t)n * top;
   float* wts = weight + (size_t)n * top;
+  float* score = z + E;
+  if (mode == 1) {
+    // scores over all outputs; what is compared is the score plus the output's correction
+    float zmax = -INFINITY;
+    for (int e = lane; e < E; e += WAVE) zmax = fmaxf(zmax, z[e]);
+    zmax = wave_max(zmax);
+    float total = 0.f;
+    for (int e = lane; e < E; e += WAVE) total += expf(z[e] - zmax);
+    total = wave_sum(total);
+    for (int e = lane; e < E; e += WAVE) {
+      const float sc = expf(z[e] - zmax) / total;
+      score[e] = sc;
+      z[e] = sc + (router_bias ? router_bias[e] : 0.f);
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    __builtin_amdgcn_wave_barrier();
+  }
   float best = 0.f, sum = 0.f;
   for (int c = 0; c < top; ++c) {
     float pv = -INFINITY;
@@ -161,7 +181,7 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const T* __restrict__ h
       pv = -INFINITY;
     }
     if (c == 0) best = pv;
-    const float w = pv == -INFINITY ? 0.f : expf(pv - best);
+    const float w = mode == 1 ? score[pick] : (pv == -INFINITY ? 0.f : expf(pv - best));
     sum += w;
     if (lane == 0) {
       mine[c] = pick;
@@ -171,14 +191,19 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const T* __restrict__ h
     __builtin_amdgcn_s_waitcnt(0);   // (the wave's own LDS write above is read by its next scan)
     __builtin_amdgcn_wave_barrier();
   }
-  if (lane == 0)
-    for (int c = 0; c < top; ++c) wts[c] = sum > 0.f ? wts[c] / sum : 0.f;
+  if (lane == 0) {
+    if (mode == 1)
+      for (int c = 0; c < top; ++c) wts[c] = wts[c] / (sum + 1e-20f);
+    else
+      for (int c = 0; c < top; ++c) wts[c] = sum > 0.f ? wts[c] / sum : 0.f;
+  }
 }
 
 // ------------------------------------------------------------------------------------------------- group
 // One workgroup: counts per expert, every expert's stretch rounded up to whole tiles, then each pair takes the next
 // free place of its expert's stretch.  sorted_pair [cap]: the pair at each place (-1: padding); pair_pos [n_pairs]:
 // each pair's place; tile_expert [cap / bm]: the expert of each tile (-1: beyond the last stretch).
+// (a pair whose expert is E or beyond, an identity expert, gets the place -1)
 __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__ chosen, int n_pairs, int E, int bm,
                                                          int* __restrict__ sorted_pair, int* __restrict__ pair_pos,
                                                          int* __restrict__ tile_expert, int cap) {
@@ -187,7 +212,8 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__
   for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = 0;
   for (int m = threadIdx.x; m < cap; m += blockDim.x) sorted_pair[m] = -1;
   __syncthreads();
-  for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) atomicAdd(&count[chosen[i]], 1);
+  for (int i = threadIdx.x; i < n_pairs; i += blockDim.x)
+    if (chosen[i] < E) atomicAdd(&count[chosen[i]], 1);
   __syncthreads();
   if (threadIdx.x == 0) {
     int at = 0;
@@ -215,6 +241,7 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__
   __syncthreads();
   for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) {
     const int e = chosen[i];
+    if (e >= E) { pair_pos[i] = -1; continue; }
     const int m = start[e] + atomicAdd(&count[e], 1);
     sorted_pair[m] = i;
     pair_pos[i] = m;
@@ -522,17 +549,23 @@ int launch_tiled(const bf16* X, long ldx, int top, const int* sorted_pair, const
 }
 
 // ------------------------------------------------------------------------------------------------- combine
+// (`self` [n, W], not null: a choice whose place is -1 is an identity expert, its result the row of `self`)
 template <typename T, bool VEC>
 __global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restrict__ pair_pos, const float* __restrict__ weight,
-                                   const T* __restrict__ shared, const float* __restrict__ sgate, T* __restrict__ out, int top, int W) {
+                                   const T* __restrict__ shared, const float* __restrict__ sgate, const T* __restrict__ self,
+                                   T* __restrict__ out, int top, int W) {
   constexpr int MOST = 8;      // choices whose places and weights a thread keeps in registers
   const int n = blockIdx.x;
   const float g = shared ? (sgate ? sgate[n] : 1.0f) : 0.f;
-  size_t at[MOST];
+  const T* at[MOST];
   float w[MOST];
+  auto row_of = [&](int s) -> const T* {
+    const int place = pair_pos[(size_t)n * top + s];
+    return (self && place < 0) ? self + (size_t)n * W : y + (size_t)place * W;
+  };
 #pragma unroll
   for (int s = 0; s < MOST; ++s) {
-    at[s] = s < top ? (size_t)pair_pos[(size_t)n * top + s] * W : 0;
+    at[s] = s < top ? row_of(s) : y;
     w[s] = s < top ? weight[(size_t)n * top + s] : 0.f;
   }
   if (VEC) {
@@ -541,12 +574,12 @@ __global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restric
 #pragma unroll
       for (int s = 0; s < MOST; ++s)
         if (s < top) {
-          const float4 r = load4f(y + at[s] + c);
+          const float4 r = load4f(at[s] + c);
           v.x = fmaf(w[s], r.x, v.x); v.y = fmaf(w[s], r.y, v.y); v.z = fmaf(w[s], r.z, v.z); v.w = fmaf(w[s], r.w, v.w);
         }
       for (int s = MOST; s < top; ++s) {
         const float ws = weight[(size_t)n * top + s];
-        const float4 r = load4f(y + (size_t)pair_pos[(size_t)n * top + s] * W + c);
+        const float4 r = load4f(row_of(s) + c);
         v.x = fmaf(ws, r.x, v.x); v.y = fmaf(ws, r.y, v.y); v.z = fmaf(ws, r.z, v.z); v.w = fmaf(ws, r.w, v.w);
       }
       if (shared) {
@@ -559,7 +592,7 @@ __global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restric
   }
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     float v = 0.f;
-    for (int s = 0; s < top; ++s) v = fmaf(weight[(size_t)n * top + s], to_float(y[(size_t)pair_pos[(size_t)n * top + s] * W + c]), v);
+    for (int s = 0; s < top; ++s) v = fmaf(weight[(size_t)n * top + s], to_float(row_of(s)[c]), v);
     if (shared) v = fmaf(g, to_float(shared[(size_t)n * W + c]), v);
     out[(size_t)n * W + c] = from_float<T>(v);
   }
@@ -573,22 +606,30 @@ GIBBS_EXPORT long gibbs_moe_capacity(int n_pairs, int E, int bm) {
 // Tiles of pairs: 16 while the matrices are streamed for few pairs each (at most 64 an expert on average), 128 beyond.
 GIBBS_EXPORT int gibbs_moe_tile(int n_pairs, int E) { return (long)n_pairs <= 64L * E ? 16 : 128; }
 
-GIBBS_EXPORT int gibbs_moe_route(const void* h, long ldh, int dtype, const float* router, const float* router_bias,
-                                 const float* shared_gate, int* chosen, float* weight, float* sgate, int n, int W, int E, int top,
-                                 hipStream_t stream) {
+// mode 0: the largest logits (+ bias), weights by the softmax over the chosen; mode 1: scores by the softmax over all E
+// outputs, the largest of score + router_bias (a correction that only the choice sees), weights the chosen scores over their sum.
+GIBBS_EXPORT int gibbs_moe_route_mode(const void* h, long ldh, int dtype, const float* router, const float* router_bias,
+                                      const float* shared_gate, int* chosen, float* weight, float* sgate, int n, int W, int E, int top,
+                                      int mode, hipStream_t stream) {
+  GIBBS_REQUIRE(mode == 0 || mode == 1, "moe_route: mode %d", mode);
   GIBBS_REQUIRE(h && router && chosen && weight && n > 0 && W > 0 && ldh >= W, "moe_route: bad operands n=%d width=%d", n, W);
   GIBBS_REQUIRE(E > 0 && E <= MOE_MAX_EXPERTS && top > 0 && top <= E, "moe_route: %d of %d experts (at most %d)", top, E, MOE_MAX_EXPERTS);
   GIBBS_REQUIRE(!shared_gate || sgate, "moe_route: a shared expert's gate needs its output");
-  const size_t lds = (size_t)E * sizeof(float);
+  const size_t lds = (size_t)E * sizeof(float) * (mode == 1 ? 2 : 1);
   // few rows: a wave per expert (and one for the shared expert's gate) up to 16 waves; many rows fill the chip with 4
   const int threads = n >= 512 ? 256 : WAVE * std::min(16, std::max(4, E + 1));
   if (dtype == GIBBS_F32)
-    moe_route_kernel<float><<<n, threads, lds, stream>>>((const float*)h, ldh, router, router_bias, shared_gate, chosen, weight, sgate, W, E, top);
+    moe_route_kernel<float><<<n, threads, lds, stream>>>((const float*)h, ldh, router, router_bias, shared_gate, chosen, weight, sgate, W, E, top, mode);
   else if (dtype == GIBBS_BF16)
-    moe_route_kernel<bf16><<<n, threads, lds, stream>>>((const bf16*)h, ldh, router, router_bias, shared_gate, chosen, weight, sgate, W, E, top);
+    moe_route_kernel<bf16><<<n, threads, lds, stream>>>((const bf16*)h, ldh, router, router_bias, shared_gate, chosen, weight, sgate, W, E, top, mode);
   else
     return gibbs_fail("moe_route: unknown dtype %d", dtype);
   GIBBS_LAUNCH_STATUS("moe_route");
+}
+GIBBS_EXPORT int gibbs_moe_route(const void* h, long ldh, int dtype, const float* router, const float* router_bias,
+                                 const float* shared_gate, int* chosen, float* weight, float* sgate, int n, int W, int E, int top,
+                                 hipStream_t stream) {
+  return gibbs_moe_route_mode(h, ldh, dtype, router, router_bias, shared_gate, chosen, weight, sgate, n, W, E, top, 0, stream);
 }
 
 GIBBS_EXPORT int gibbs_moe_group(const int* chosen, int n_pairs, int E, int bm, int* sorted_pair, int* pair_pos, int* tile_expert,
@@ -647,11 +688,16 @@ GIBBS_EXPORT int gibbs_moe_gemm(const void* X, long ldx, int top, const int* sor
 // out[n] = sum_c weight[n][c] y[pair_pos[n * top + c]] + sgate[n] shared[n]  (shared null: no shared expert; sgate null: 1).
 GIBBS_EXPORT int gibbs_moe_combine(const void* y, const int* pair_pos, const float* weight, const void* shared, const float* sgate,
                                    void* out, int dtype, int n, int top, int W, hipStream_t stream) {
+  return gibbs_moe_combine_self(y, pair_pos, weight, shared, sgate, nullptr, out, dtype, n, top, W, stream);
+}
+// self [n, W] (null: none): the rows themselves, which a choice without a place (-1: an identity expert) stands for.
+GIBBS_EXPORT int gibbs_moe_combine_self(const void* y, const int* pair_pos, const float* weight, const void* shared, const float* sgate,
+                                        const void* self, void* out, int dtype, int n, int top, int W, hipStream_t stream) {
   GIBBS_REQUIRE(y && pair_pos && weight && out && n > 0 && top > 0 && W > 0, "moe_combine: bad operands n=%d top=%d width=%d", n, top, W);
   const size_t bytes = dtype == GIBBS_F32 ? 16 : 8;
-  const bool vec = W % 4 == 0 && ((uintptr_t)y % bytes) == 0 && ((uintptr_t)shared % bytes) == 0 && ((uintptr_t)out % bytes) == 0;
+  const bool vec = W % 4 == 0 && ((uintptr_t)y % bytes) == 0 && ((uintptr_t)shared % bytes) == 0 && ((uintptr_t)out % bytes) == 0 && ((uintptr_t)self % bytes) == 0;
   const int threads = vec ? (W >= 4096 ? 1024 : (W >= 1024 ? 256 : 64)) : (W >= 1024 ? 256 : 64);
-#define MOE_COMBINE(T, V) moe_combine_kernel<T, V><<<n, threads, 0, stream>>>((const T*)y, pair_pos, weight, (const T*)shared, sgate, (T*)out, top, W)
+#define MOE_COMBINE(T, V) moe_combine_kernel<T, V><<<n, threads, 0, stream>>>((const T*)y, pair_pos, weight, (const T*)shared, sgate, (const T*)self, (T*)out, top, W)
   if (dtype == GIBBS_F32) {
     if (vec) MOE_COMBINE(float, true); else MOE_COMBINE(float, false);
   } else if (dtype == GIBBS_BF16) {

@@ -14,6 +14,13 @@
 // value size: heads may be stored wider, zeros behind their vt channels), and a later layer mixes them into its
 // own before they are cached,  v <- (1 - lambda) v + lambda v_published,  lambda one number on the device.  The
 // mix is float32 arithmetic (the layer's own value with its bias still unrounded), rounded once.
+//
+// Further options (`gibbs_qkv_prepare_full`): q and k heads divided by their root mean square and multiplied by a gain
+// [norm_dim] before the rotation (the mean over the first norm_dim channels of a head, which may be stored wider with
+// zeros behind them); values that are the keys as projected (`v_from_k`: rows hold no values, the key's wave writes the
+// unnormed, unrotated key into the value page); and values turned by their position over all of their first `v_rot`
+// channels, pairs in the same layout, angle float(pos) * v_inv_freq[m], before they are cached.  `gibbs_attention_finish`
+// is the other end of that: the heads' outputs turned back by the query's position and multiplied by sigmoid(gate).
 #include "common.h"
 #include "lane8.h"
 
@@ -35,6 +42,13 @@ struct QkvPrepareArgs {
   int max_pages, page_size, num_pages;
   int nh, nkv, hd, vd;
   long ld;
+  const float* q_gain;     // [norm_dim] or null: q heads are RMS-normed with this gain before the rotation
+  const float* k_gain;     // the same for k heads
+  float qk_eps;
+  int norm_dim;            // channels of a head that the norm's mean runs over
+  int v_from_k;            // the values are the keys as projected: rows are [q | k | ...], no value heads
+  const float* v_inv_freq; // [v_rot / 2] or null: values are turned by their position over their first v_rot channels
+  int v_rot;
 };
 
 template <typename T>
@@ -43,7 +57,7 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(T* __restrict__ rows, 
   const int n = blockIdx.x;
   const int hs = blockIdx.y * (blockDim.x / WAVE) + threadIdx.x / WAVE;
   const int lane = threadIdx.x % WAVE;
-  if (hs >= a.nh + 2 * a.nkv) return;
+  if (hs >= a.nh + (a.v_from_k ? 1 : 2) * a.nkv) return;
   const bool is_q = hs < a.nh, is_k = !is_q && hs < a.nh + a.nkv;
   const int g = is_q ? hs : (is_k ? hs - a.nh : hs - a.nh - a.nkv);
   const int size = (is_q || is_k) ? a.hd : a.vd;
@@ -57,12 +71,43 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(T* __restrict__ rows, 
     if (page >= 0 && page < a.num_pages)   // (the host never asks for another; never write outside the pool)
       page_dst = (is_k ? kpages : vpages) + (((size_t)page * a.nkv + g) * a.page_size + p % a.page_size) * size;
   }
-  auto value = [&](int e) -> float { return bias ? to_float(src[e]) + bias[e] : to_float(src[e]); };
+  auto raw_value = [&](int e) -> float { return bias ? to_float(src[e]) + bias[e] : to_float(src[e]); };
   auto put = [&](int e, float v) {
     const T r = from_float<T>(v);
     src[e] = r;
     if (page_dst) page_dst[e] = r;
   };
+  if (is_k && a.v_from_k && vpages) {
+    // the value of this position is the key as projected (vd channels of it), before norm and rotation
+    const int page = a.table[(size_t)a.row_req[n] * a.max_pages + p / a.page_size];
+    if (page >= 0 && page < a.num_pages) {
+      T* vdst = vpages + (((size_t)page * a.nkv + g) * a.page_size + p % a.page_size) * a.vd;
+      for (int e = lane; e < a.vd; e += WAVE) vdst[e] = from_float<T>(e < a.hd ? raw_value(e) : 0.f);
+    }
+  }
+  if (!is_q && !is_k && a.v_inv_freq) {
+    const int vh = a.v_rot / 2;
+    for (int j = lane; j < vh; j += WAVE) {
+      const int i0 = a.variant == ROPE_HALF_SPLIT ? j : 2 * j;
+      const int i1 = a.variant == ROPE_HALF_SPLIT ? j + vh : 2 * j + 1;
+      const float x0 = raw_value(i0), x1 = raw_value(i1);
+      float c, s;
+      rope_cos_sin((float)p * a.v_inv_freq[j], &c, &s);
+      put(i0, x0 * c - x1 * s);
+      put(i1, x1 * c + x0 * s);
+    }
+    for (int e = a.v_rot + lane; e < size; e += WAVE) put(e, raw_value(e));
+    return;
+  }
+  // q and k heads: x / sqrt(mean(x^2) + eps) * gain over the head's first norm_dim channels, before the rotation
+  const float* gain = is_q ? a.q_gain : (is_k ? a.k_gain : nullptr);
+  float inv = 1.0f;
+  if (gain) {
+    float ss = 0.f;
+    for (int e = lane; e < a.norm_dim; e += WAVE) { const float x = raw_value(e); ss = fmaf(x, x, ss); }
+    inv = 1.0f / sqrtf(wave_sum(ss) / (float)a.norm_dim + a.qk_eps);
+  }
+  auto value = [&](int e) -> float { return gain ? (e < a.norm_dim ? raw_value(e) * inv * gain[e] : 0.f) : raw_value(e); };
   if (!is_q && !is_k) {
     const float lam = a.keep_mode == KEEP_MIX ? *a.lambda : 0.f;
     T* kept = a.keep_mode != KEEP_NONE ? keep + ((size_t)n * a.nkv + g) * a.vt : nullptr;
@@ -196,23 +241,57 @@ __global__ __launch_bounds__(256) void qkv_prepare_bf16x8_kernel(bf16* __restric
   put(j0, y0);
   put(j0 + half, y1);
 }
+// The heads' outputs att [N, nh * vd] (row stride ldo), in place: each head turned back by its row's position over its
+// first v_rot channels (pair m by -pos * v_inv_freq[m]; null: not turned), then multiplied element by element with
+// sigmoid(gate[n, h * gate_head + c]) (gate rows of stride ld_gate in the same type, c < vt; null: no gate).  float32 arithmetic.
+template <typename T>
+__global__ __launch_bounds__(256) void attention_finish_kernel(T* __restrict__ att, long ldo, const T* __restrict__ gate, long ld_gate,
+                                                               int gate_head, const int* __restrict__ pos, const float* __restrict__ v_inv_freq,
+                                                               int v_rot, int variant, int nh, int vd, int vt) {
+  const int n = blockIdx.x;
+  const int h = blockIdx.y * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+  const int lane = threadIdx.x % WAVE;
+  if (h >= nh) return;
+  T* o = att + (size_t)n * ldo + (size_t)h * vd;
+  const T* g = gate ? gate + (size_t)n * ld_gate + (size_t)h * gate_head : nullptr;
+  auto gated = [&](int e, float v) -> float { return (g && e < vt) ? v / (1.0f + expf(-to_float(g[e]))) : v; };
+  const int vh = v_inv_freq ? v_rot / 2 : 0;
+  const float p = (float)pos[n];
+  for (int j = lane; j < vh; j += WAVE) {
+    const int i0 = variant == ROPE_HALF_SPLIT ? j : 2 * j;
+    const int i1 = variant == ROPE_HALF_SPLIT ? j + vh : 2 * j + 1;
+    const float x0 = to_float(o[i0]), x1 = to_float(o[i1]);
+    float c, s;
+    rope_cos_sin(p * v_inv_freq[j], &c, &s);
+    o[i0] = from_float<T>(gated(i0, x0 * c + x1 * s));      // (the turn by -angle)
+    o[i1] = from_float<T>(gated(i1, x1 * c - x0 * s));
+  }
+  if (g)
+    for (int e = 2 * vh + lane; e < vd; e += WAVE) o[e] = from_float<T>(gated(e, to_float(o[e])));
+}
 }  // namespace
 
 // keep_mode: 0 none, 1 the values are published into `keep`, 2 `keep` is mixed into the values with *lambda.
-GIBBS_EXPORT int gibbs_qkv_prepare(void* rows, long ld, void* kpages, void* vpages, int dtype, const float* bias,
-                                   const float* inv_freq, int rot, int variant, const float* cs_table, int table_len,
-                                   void* keep, int keep_mode, int vt, const float* lambda, const int* pos, const int* row_req,
-                                   const int* table, int max_pages, int page_size, int num_pages, int n_rows, int nh, int nkv,
-                                   int hd, int vd, hipStream_t stream) {
+GIBBS_EXPORT int gibbs_qkv_prepare_full(void* rows, long ld, void* kpages, void* vpages, int dtype, const float* bias,
+                                        const float* inv_freq, int rot, int variant, const float* cs_table, int table_len,
+                                        void* keep, int keep_mode, int vt, const float* lambda, const int* pos, const int* row_req,
+                                        const int* table, int max_pages, int page_size, int num_pages, int n_rows, int nh, int nkv,
+                                        int hd, int vd, const float* q_gain, const float* k_gain, float qk_eps, int norm_dim,
+                                        int v_from_k, const float* v_inv_freq, int v_rot, hipStream_t stream) {
   GIBBS_REQUIRE(rows && pos && n_rows > 0 && nh > 0 && nkv > 0 && hd > 0 && vd > 0, "qkv_prepare: bad operands rows=%d heads=%d kv=%d", n_rows, nh, nkv);
-  GIBBS_REQUIRE(ld >= (long)(nh + nkv) * hd + (long)nkv * vd, "qkv_prepare: rows of %ld values cannot hold q, k and v", ld);
+  GIBBS_REQUIRE(ld >= (long)(nh + nkv) * hd + (v_from_k ? 0 : (long)nkv * vd), "qkv_prepare: rows of %ld values cannot hold q, k and v", ld);
   GIBBS_REQUIRE(!kpages || (vpages && row_req && table && max_pages > 0 && page_size > 0 && num_pages > 0), "qkv_prepare: pages without their table");
   GIBBS_REQUIRE(!inv_freq || (rot > 0 && rot % 2 == 0 && rot <= hd), "qkv_prepare: %d rotated channels of a head of %d", rot, hd);
   GIBBS_REQUIRE(keep_mode == KEEP_NONE || (keep && vt > 0 && vt <= vd && (keep_mode == KEEP_PUBLISH || (keep_mode == KEEP_MIX && lambda))),
                 "qkv_prepare: value mixing needs the published values and its weight");
+  GIBBS_REQUIRE(!(q_gain || k_gain) || (norm_dim > 0 && norm_dim <= hd), "qkv_prepare: a norm over %d channels of a head of %d", norm_dim, hd);
+  GIBBS_REQUIRE(!v_from_k || (keep_mode == KEEP_NONE && !v_inv_freq), "qkv_prepare: values that are the keys are neither mixed nor turned");
+  GIBBS_REQUIRE(!v_inv_freq || (v_rot > 0 && v_rot % 2 == 0 && v_rot <= vd && keep_mode == KEEP_NONE), "qkv_prepare: %d turned channels of a value head of %d", v_rot, vd);
   QkvPrepareArgs a{bias, inv_freq, inv_freq ? rot : 0, variant, (const float2*)cs_table, cs_table && inv_freq ? table_len : 0, lambda, keep_mode, vt,
-                   pos, row_req, table, max_pages, page_size, num_pages, nh, nkv, hd, vd, ld};
-  const bool x8 = dtype == GIBBS_BF16 && hd % 8 == 0 && vd % 8 == 0 && ld % 8 == 0 && ((uintptr_t)rows % 16) == 0 && (!inv_freq || (variant == ROPE_HALF_SPLIT && rot % 16 == 0)) &&
+                   pos, row_req, table, max_pages, page_size, num_pages, nh, nkv, hd, vd, ld, q_gain, k_gain, qk_eps, norm_dim, v_from_k,
+                   v_inv_freq, v_inv_freq ? v_rot : 0};
+  const bool plain_options = !q_gain && !k_gain && !v_from_k && !v_inv_freq;
+  const bool x8 = plain_options && dtype == GIBBS_BF16 && hd % 8 == 0 && vd % 8 == 0 && ld % 8 == 0 && ((uintptr_t)rows % 16) == 0 && (!inv_freq || (variant == ROPE_HALF_SPLIT && rot % 16 == 0)) &&
                   (!bias || ((uintptr_t)bias % 16) == 0) && (keep_mode == KEEP_NONE || (vt % 8 == 0 && ((uintptr_t)keep % 16) == 0)) &&
                   (!kpages || (((uintptr_t)kpages % 16) == 0 && ((uintptr_t)vpages % 16) == 0));
   if (x8) {
@@ -232,4 +311,31 @@ GIBBS_EXPORT int gibbs_qkv_prepare(void* rows, long ld, void* kpages, void* vpag
   else
     return gibbs_fail("qkv_prepare: unknown dtype %d", dtype);
   GIBBS_LAUNCH_STATUS("qkv_prepare");
+}
+GIBBS_EXPORT int gibbs_qkv_prepare(void* rows, long ld, void* kpages, void* vpages, int dtype, const float* bias,
+                                   const float* inv_freq, int rot, int variant, const float* cs_table, int table_len,
+                                   void* keep, int keep_mode, int vt, const float* lambda, const int* pos, const int* row_req,
+                                   const int* table, int max_pages, int page_size, int num_pages, int n_rows, int nh, int nkv,
+                                   int hd, int vd, hipStream_t stream) {
+  return gibbs_qkv_prepare_full(rows, ld, kpages, vpages, dtype, bias, inv_freq, rot, variant, cs_table, table_len, keep, keep_mode, vt, lambda,
+                                pos, row_req, table, max_pages, page_size, num_pages, n_rows, nh, nkv, hd, vd, nullptr, nullptr, 0.f, 0, 0,
+                                nullptr, 0, stream);
+}
+
+GIBBS_EXPORT int gibbs_attention_finish(void* att, long ldo, const void* gate, long ld_gate, int gate_head, int dtype, const int* pos,
+                                        const float* v_inv_freq, int v_rot, int variant, int n_rows, int nh, int vd, int vt,
+                                        hipStream_t stream) {
+  GIBBS_REQUIRE(att && n_rows > 0 && nh > 0 && vd > 0 && vt > 0 && vt <= vd && ldo >= (long)nh * vd, "attention_finish: bad operands rows=%d heads=%d vd=%d", n_rows, nh, vd);
+  GIBBS_REQUIRE(!v_inv_freq || (pos && v_rot > 0 && v_rot % 2 == 0 && v_rot <= vd), "attention_finish: %d turned channels of a head of %d", v_rot, vd);
+  GIBBS_REQUIRE(!gate || (gate_head >= vt && ld_gate >= (long)nh * gate_head), "attention_finish: gate rows too short");
+  if (!gate && !v_inv_freq) return 0;
+  const int per_block = 4;
+  const dim3 grid(n_rows, ceil_div(nh, per_block));
+  if (dtype == GIBBS_F32)
+    attention_finish_kernel<float><<<grid, per_block * WAVE, 0, stream>>>((float*)att, ldo, (const float*)gate, ld_gate, gate_head, pos, v_inv_freq, v_rot, variant, nh, vd, vt);
+  else if (dtype == GIBBS_BF16)
+    attention_finish_kernel<bf16><<<grid, per_block * WAVE, 0, stream>>>((bf16*)att, ldo, (const bf16*)gate, ld_gate, gate_head, pos, v_inv_freq, v_rot, variant, nh, vd, vt);
+  else
+    return gibbs_fail("attention_finish: unknown dtype %d", dtype);
+  GIBBS_LAUNCH_STATUS("attention_finish");
 }

@@ -18,28 +18,34 @@ __device__ __forceinline__ float activate_gate(float z, int act) {   // 0: silu,
 }
 
 // ------------------------------------------------------------------------------------------------ short causal convolution
-// y[n, c] = silu(sum_j taps[c, j] * x[t - (K-1) + j, c]): the last tap is the current token's; inputs before the
-// step's first row come from the request's state (its last K-1 inputs, oldest first; zeros at a sequence's start).
-template <typename T>
-__global__ void causal_conv_silu_kernel(const T* __restrict__ in, long ld, const float* __restrict__ taps,
+// y[n, c] = act(sum_j taps[c, j] * x[t - (K-1) + j, c] + bias[c]) (+ x[t, c]): the last tap is the current token's; inputs
+// before the step's first row come from the request's state (its last K-1 inputs, oldest first; zeros at a sequence's
+// start).  act: silu or none; `residual`: the input itself is added to the result (a convolution beside the identity).
+enum { CONV_ACT_NONE = 0, CONV_ACT_SILU = 1 };
+template <typename T, typename TO>
+__global__ void causal_conv_silu_kernel(const T* __restrict__ in, long ld, const float* __restrict__ taps, const float* __restrict__ bias,
                                         float* __restrict__ state, long slot_stride, const int* __restrict__ row_req,
-                                        const int* __restrict__ cu, const int* __restrict__ slot, float* __restrict__ out,
-                                        int C, int K, int shift_state) {
+                                        const int* __restrict__ cu, const int* __restrict__ slot, TO* __restrict__ out, long ld_out,
+                                        int C, int K, int shift_state, int act, int residual) {
   const int n = blockIdx.x;
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= C) return;
   const int r = row_req[n], first = cu[r], t = n - first;
   float* st = state + (size_t)slot[r] * slot_stride;
-  float acc = 0.f;
+  float acc = 0.f, own = 0.f;
   for (int j = 0; j < K; ++j) {
     const int tt = t - (K - 1) + j;
     const float xv = tt >= 0 ? to_float(in[(size_t)(first + tt) * ld + c]) : st[(size_t)(K - 1 + tt) * C + c];
     acc = fmaf(taps[(size_t)c * K + j], xv, acc);
+    own = xv;
     // every request brings one row (shift_state): this thread is the only one that reads or writes the request's
     // inputs of this channel, so it moves them on itself (entry j - 1 has been read already)
     if (shift_state && j >= 1) st[(size_t)(j - 1) * C + c] = xv;
   }
-  out[(size_t)n * C + c] = acc * sigmoid_f(acc);
+  if (bias) acc += bias[c];
+  if (act == CONV_ACT_SILU) acc = acc * sigmoid_f(acc);
+  if (residual) acc += own;
+  out[(size_t)n * ld_out + c] = from_float<TO>(acc);
 }
 
 // The state after the step: the last K-1 inputs of the request (what the step brought, and before that what
@@ -112,7 +118,7 @@ __global__ __launch_bounds__(64) void delta_prep_kernel(DeltaPrepArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------------ the recurrences
-enum { RULE_DELTA = 0, RULE_OUTER = 1 };
+enum { RULE_DELTA = 0, RULE_OUTER = 1, RULE_SSD = 2 };
 struct RecurrenceArgs {
   const void* q;       // delta: unit q * scale; outer: the receptance r.  [N, G*D]
   const void* k;       // [N, G*D]
@@ -139,6 +145,7 @@ struct RecurrenceArgs {
 // With M the state [D, V], ' for transposed and .* for element by element along the key channels:
 //   delta:  M = decay * M;  w = beta * (v - M' k);  M = M + k w';  read = M' q
 //   outer:  read = (M + (bonus .* k) v')' r;  M = decay .* M (row by row) + k v'
+//   ssd:    M = decay * M + k v';  read = M' q      (the delta rule without its correction and with beta = 1)
 // CH: the decay is one per key channel (always so for the outer rule); else one per head.
 template <typename TIn, int RULE, int DPT, int PARTS, bool CH>
 __global__ __launch_bounds__(64) void recurrence_kernel(RecurrenceArgs a) {
@@ -184,10 +191,10 @@ __global__ __launch_bounds__(64) void recurrence_kernel(RecurrenceArgs a) {
       const int idx = e * WAVE + lane, t = idx / COLS, jj = blockIdx.z * COLS + idx % COLS;
       rv[e] = (t < nt && jj < V) ? to_float(v[(size_t)(first + t0 + t) * a.ldv + (size_t)h * V + jj]) : 0.f;
     }
-    if (RULE == RULE_DELTA && lane < TOK) {
+    if (RULE != RULE_OUTER && lane < TOK) {
       const bool live = lane < nt;
       const size_t row = (size_t)(first + t0 + (live ? lane : 0));
-      rb = live ? a.beta[row * a.H + h] : 0.f;
+      rb = (live && RULE == RULE_DELTA) ? a.beta[row * a.H + h] : 0.f;
       rg = (live && !a.per_channel) ? a.decay[row * a.H + h] : 1.f;
     }
   };
@@ -204,7 +211,7 @@ __global__ __launch_bounds__(64) void recurrence_kernel(RecurrenceArgs a) {
       const int idx = e * WAVE + lane;
       if (idx < TOK * COLS) sv[idx / COLS][idx % COLS] = rv[e];
     }
-    if (RULE == RULE_DELTA && lane < TOK) {
+    if (RULE != RULE_OUTER && lane < TOK) {
       sb[lane] = rb;
       sg[lane] = rg;
     }
@@ -244,11 +251,19 @@ __global__ __launch_bounds__(64) void recurrence_kernel(RecurrenceArgs a) {
       }
       v_ = sv[t][col];
       b_ = RULE == RULE_DELTA ? sb[t] : 0.f;
-      g_ = RULE == RULE_DELTA ? sg[t] : 1.f;
+      g_ = RULE != RULE_OUTER ? sg[t] : 1.f;
     };
     auto step = [&](int t, const float (&k_)[DPT], const float (&q_)[DPT], const float (&d_)[DPT], float v_, float b_, float g_) {
       float o0 = 0.f, o1 = 0.f;
-      if (RULE == RULE_DELTA) {
+      if (RULE == RULE_SSD) {
+#pragma unroll
+        for (int ii = 0; ii < DPT; ii += 2) {
+          S[ii] = fmaf(channel_decay ? d_[ii] : g_, S[ii], k_[ii] * v_);
+          S[ii + 1] = fmaf(channel_decay ? d_[ii + 1] : g_, S[ii + 1], k_[ii + 1] * v_);
+          o0 = fmaf(S[ii], q_[ii], o0);
+          o1 = fmaf(S[ii + 1], q_[ii + 1], o1);
+        }
+      } else if (RULE == RULE_DELTA) {
         float dot0 = 0.f, dot1 = 0.f;
 #pragma unroll
         for (int ii = 0; ii < DPT; ii += 2) {
@@ -380,22 +395,37 @@ __global__ void double_exp_decay_kernel(float* __restrict__ z, const float* __re
     else return gibbs_fail(what ": unknown dtype %d", (dtype)); \
   } while (0)
 
-GIBBS_EXPORT int gibbs_causal_conv_silu(const void* in, long ld, int dtype, const float* taps, float* state, long slot_stride,
-                                        const int* row_req, const int* cu, const int* slot, float* out, int n_rows, int n_req,
-                                        int C, int K, int update_state, int single_rows, hipStream_t stream) {
+// The general entry point: an optional bias [C], act 0 none / 1 silu, `residual` (the input is added to the result), and the
+// result as float32 (out_f32) or in the input's type, in rows of ld_out values.  `in` and `out` must not overlap.
+GIBBS_EXPORT int gibbs_causal_conv(const void* in, long ld, int dtype, const float* taps, const float* bias, float* state, long slot_stride,
+                                   const int* row_req, const int* cu, const int* slot, void* out, int out_f32, long ld_out, int n_rows,
+                                   int n_req, int C, int K, int act, int residual, int update_state, int single_rows, hipStream_t stream) {
   // single_rows: every request brings exactly one row (a step of decoded tokens): the state moves on in the same kernel
   const int shift = update_state && single_rows && K > 1 && n_rows == n_req;
-  GIBBS_REQUIRE(in && taps && state && out && n_rows > 0 && n_req > 0 && C > 0 && K >= 1 && ld >= C && slot_stride >= (long)(K - 1) * C,
+  GIBBS_REQUIRE(in && taps && state && out && n_rows > 0 && n_req > 0 && C > 0 && K >= 1 && ld >= C && ld_out >= C && slot_stride >= (long)(K - 1) * C,
                 "causal_conv: bad operands rows=%d requests=%d C=%d K=%d", n_rows, n_req, C, K);
   const dim3 rows(n_rows, ceil_div(C, 256)), reqs(n_req, ceil_div(C, 256));
-  BY_DTYPE(dtype, "causal_conv",
-           (causal_conv_silu_kernel<float><<<rows, 256, 0, stream>>>((const float*)in, ld, taps, state, slot_stride, row_req, cu, slot, out, C, K, shift)),
-           (causal_conv_silu_kernel<bf16><<<rows, 256, 0, stream>>>((const bf16*)in, ld, taps, state, slot_stride, row_req, cu, slot, out, C, K, shift)));
+#define CONV_ARGS taps, bias, state, slot_stride, row_req, cu, slot
+  if (out_f32 || dtype == GIBBS_F32)
+    BY_DTYPE(dtype, "causal_conv",
+             (causal_conv_silu_kernel<float, float><<<rows, 256, 0, stream>>>((const float*)in, ld, CONV_ARGS, (float*)out, ld_out, C, K, shift, act, residual)),
+             (causal_conv_silu_kernel<bf16, float><<<rows, 256, 0, stream>>>((const bf16*)in, ld, CONV_ARGS, (float*)out, ld_out, C, K, shift, act, residual)));
+  else if (dtype == GIBBS_BF16)
+    causal_conv_silu_kernel<bf16, bf16><<<rows, 256, 0, stream>>>((const bf16*)in, ld, CONV_ARGS, (bf16*)out, ld_out, C, K, shift, act, residual);
+  else
+    return gibbs_fail("causal_conv: unknown dtype %d", dtype);
+#undef CONV_ARGS
   if (update_state && K > 1 && !shift)
     BY_DTYPE(dtype, "causal_conv",
              (causal_conv_state_kernel<float><<<reqs, 256, 0, stream>>>((const float*)in, ld, state, slot_stride, cu, slot, C, K)),
              (causal_conv_state_kernel<bf16><<<reqs, 256, 0, stream>>>((const bf16*)in, ld, state, slot_stride, cu, slot, C, K)));
   GIBBS_LAUNCH_STATUS("causal_conv");
+}
+GIBBS_EXPORT int gibbs_causal_conv_silu(const void* in, long ld, int dtype, const float* taps, float* state, long slot_stride,
+                                        const int* row_req, const int* cu, const int* slot, float* out, int n_rows, int n_req,
+                                        int C, int K, int update_state, int single_rows, hipStream_t stream) {
+  return gibbs_causal_conv(in, ld, dtype, taps, nullptr, state, slot_stride, row_req, cu, slot, out, 1, C, n_rows, n_req, C, K, 1, 0,
+                           update_state, single_rows, stream);
 }
 
 GIBBS_EXPORT int gibbs_delta_prep(float* q, float* k, long ldqk, const void* beta_raw, const void* a_head, long ld_raw, int dtype,
@@ -417,6 +447,42 @@ int check_recurrence(const char* what, int n_req, int H, int G, int D, int V, lo
   return 0;
 }
 }  // namespace
+
+// What the state-space rule reads, from the convolved rows xbc [N, ld_x] (float32: x [H*V] first) and the projected rows'
+// dt entries (raw [N, ld_raw] in the activation type, H values from column 0 of `dt_raw`):
+//   dt = softplus(dt_raw + dt_bias);  decay = exp(-exp(a_log) dt);  xdt = dt x      (all float32)
+template <typename T>
+__global__ void ssd_prep_kernel(const float* __restrict__ xbc, long ld_x, const T* __restrict__ dt_raw, long ld_raw,
+                                const float* __restrict__ dt_bias, const float* __restrict__ a_log, float* __restrict__ decay,
+                                float* __restrict__ xdt, int H, int V) {
+  const int n = blockIdx.x, h = blockIdx.y;
+  const float dt = softplus_f(to_float(dt_raw[(size_t)n * ld_raw + h]) + dt_bias[h]);
+  if (threadIdx.x == 0) decay[(size_t)n * H + h] = expf(-expf(a_log[h]) * dt);
+  for (int j = threadIdx.x; j < V; j += blockDim.x) xdt[(size_t)n * H * V + (size_t)h * V + j] = dt * xbc[(size_t)n * ld_x + (size_t)h * V + j];
+}
+GIBBS_EXPORT int gibbs_ssd_prep(const float* xbc, long ld_x, const void* dt_raw, long ld_raw, int dtype, const float* dt_bias,
+                                const float* a_log, float* decay, float* xdt, int n_rows, int H, int V, hipStream_t stream) {
+  GIBBS_REQUIRE(xbc && dt_raw && dt_bias && a_log && decay && xdt && n_rows > 0 && H > 0 && V > 0 && ld_x >= (long)H * V && ld_raw >= H,
+                "ssd_prep: bad operands rows=%d heads=%d V=%d", n_rows, H, V);
+  GIBBS_REQUIRE(H <= 65535, "ssd_prep: too many heads (%d)", H);
+  const dim3 grid(n_rows, H);
+  BY_DTYPE(dtype, "ssd_prep",
+           (ssd_prep_kernel<float><<<grid, WAVE, 0, stream>>>(xbc, ld_x, (const float*)dt_raw, ld_raw, dt_bias, a_log, decay, xdt, H, V)),
+           (ssd_prep_kernel<bf16><<<grid, WAVE, 0, stream>>>(xbc, ld_x, (const bf16*)dt_raw, ld_raw, dt_bias, a_log, decay, xdt, H, V)));
+  GIBBS_LAUNCH_STATUS("ssd_prep");
+}
+
+// The decayed outer-product rule with one decay per head and the read-out after the write (see recurrence_kernel): the
+// recurrence of a state-space mixer, M [D, V] with D the state size: k = B, q = C (G groups of D), v = dt x.  All float32.
+GIBBS_EXPORT int gibbs_ssd_rule(const float* q, const float* k, long ldqk, const float* v, long ldv, const float* decay, float* state,
+                                long slot_stride, const int* cu, const int* slot, float* out, int n_req, int H, int G, int D, int V,
+                                hipStream_t stream) {
+  GIBBS_REQUIRE(q && k && v && decay && state && cu && slot && out && ldqk >= (long)G * D && ldv >= (long)H * V, "ssd_rule: null operand or short rows");
+  if (check_recurrence("ssd_rule", n_req, H, G, D, V, slot_stride)) return 1;
+  RecurrenceArgs a{q, k, v, ldqk, ldqk, ldv, decay, 0, nullptr, nullptr, state, slot_stride, cu, slot, out, H, G, D, V};
+  launch_recurrence<float, RULE_SSD>(a, n_req, stream);
+  GIBBS_LAUNCH_STATUS("ssd_rule");
+}
 
 // The gated delta rule over a ragged batch; q, k (unit vectors, q scaled), v, beta, decay float32.
 GIBBS_EXPORT int gibbs_delta_rule(const float* q, const float* k, long ldqk, const float* v, long ldv, const float* beta, const float* decay,

@@ -292,6 +292,9 @@ struct NormPart {
   virtual void* run_streams(Exec& e, const float* x, int streams, const float* coef, const int* rows, int n_out) const;
   // a plain RMS norm with its gain (null: none) and eps, for kernels that apply it beside their own work
   virtual bool plain_rms(const float** gain, float* eps) const { return false; }
+  // an RMS norm in groups (1: a plain one) with its gain, for the kernel that norms a result into the stream and the
+  // stream for the next sublayer in one pass
+  virtual bool group_rms(const float** gain, float* eps, int* groups) const { return false; }
   // a norm that the streams' kernels apply themselves: its kind there (0 root mean square, 1 layer norm) and operands
   virtual bool for_streams(int* kind, const float** gain, const float** bias, float* eps) const { return false; }
 };
@@ -337,12 +340,13 @@ struct Plan {
   bool plain_embedding() const { return embed_scale == 1.0f && !embed_inv_freq && !reinjects && !table_sums(); }
   bool reinjects = false;              // the program adds the embedding's output into the stream again
   Matrix head;
+  float logit_softcap = 0.f;   // > 0: logits <- cap * tanh(logits / cap)
   int tail = -1;            // the norm in front of the head
   int fused_rows = FUSED_ROWS;   // steps of at most this many decoded tokens take the fused decode kernels
   int own_gemm = 0;         // products above the few-row kernels' range: 0 the library's, 1 the tiled kernel
   std::vector<std::unique_ptr<NormPart>> norms;
   std::vector<std::unique_ptr<Body>> bodies;
-  enum { OP_HALF, OP_NORM, OP_BODY, OP_ADD, OP_DROP, OP_NORM_DELTA, OP_REINJECT, OP_ADD_NORMED, OP_STREAMS_NORM, OP_STREAMS_ADD };
+  enum { OP_HALF, OP_NORM, OP_BODY, OP_ADD, OP_DROP, OP_NORM_DELTA, OP_REINJECT, OP_ADD_NORMED, OP_STREAMS_NORM, OP_STREAMS_ADD, OP_ROWS };
   struct Op {
     int kind, norm, body, value;   // value: what a body reads, an add adds, a drop drops
     int result;                    // the value that a norm or a body makes
@@ -456,6 +460,30 @@ struct RmsNorm : NormPart {
     return out;
   }
 };
+// RMS norm in `groups` equal consecutive parts of the row, each divided by its own root mean square; the gain over the whole row.
+struct GroupRmsNorm : NormPart {
+  const float* gain = nullptr;
+  float eps = 0.f;
+  int groups = 1;
+  void* run(Exec& e, float* x, Pending& pending, const int* rows, int n_out) const override {
+    const int H = e.p.hidden;
+    e.settle(x, pending);
+    void* out = e.take((long)n_out * H * e.esize);
+    RUN(e, gibbs_group_rmsnorm(x, nullptr, 0, 0, nullptr, 0.f, 0, gain, eps, groups, out, e.p.dtype, rows, n_out, H, e.a.stream));
+    return out;
+  }
+  bool group_rms(const float** g, float* ep, int* gr) const override {
+    *g = gain; *ep = eps; *gr = groups;
+    return true;
+  }
+  bool add_normed(Exec& e, float* x, Pending delta) const override {
+    const int N = e.a.n_rows, H = e.p.hidden;
+    RUN(e, gibbs_group_rmsnorm(x, delta.data, std::max(delta.parts, 1), (long)N * H, gain, eps, groups, nullptr, 0.f, 0, nullptr, e.p.dtype, nullptr,
+                               N, H, e.a.stream));
+    e.give(delta.data);
+    return true;
+  }
+};
 // Layer norm with gain and bias: (x - mean) / sqrt(mean((x - mean)^2) + eps) * gain + bias, all in float32.
 struct LayerNorm : NormPart {
   const float* gain = nullptr;
@@ -541,6 +569,8 @@ struct PagedAttention {
   const float* bias_t;    // the same as [nh, bias_len] divided by the scale: what the matrix-core kernels add to raw scores
   int bias_len;
   const float* sink;      // [nh]: a term exp(sink[h]) in the softmax's denominator without key or value
+  int chunk = 0;          // > 0: a row sees the keys of its own stretch of `chunk` positions (counted from 0) instead of a window
+  float softcap = 0.f;    // > 0: scores are capped as softcap * tanh(s / softcap)
 };
 void decode_attention(Exec& e, const PagedAttention& t, const void* q, long ldq, int n_rows, const int* pos, const int* row_req, void* o) {
   int n_splits, waves;
@@ -561,7 +591,8 @@ void* attend_prepared(Exec& e, const PagedAttention& t, void* raw, long ldq, lon
   // the matrix-core kernels take rows that are prepared (whatever prepared them), keys and values of one head
   // size, and a bias on the scores as a table over the distance (no slopes)
   const bool matrix_sizes = t.hd % 16 == 0 && t.hd <= 128;
-  const bool fast_bf16 = e.bf16_run && !t.slopes && t.vd == t.hd && (!t.bias || (t.bias_t && matrix_sizes)) && (!t.sink || t.scale > 0.f);
+  const bool fast_bf16 = e.bf16_run && !t.slopes && t.vd == t.hd && (!t.bias || (t.bias_t && matrix_sizes)) && (!t.sink || t.scale > 0.f) &&
+                         t.chunk == 0 && t.softcap == 0.f;
   if (fast_bf16 && a.max_q > 1 && matrix_sizes) {
     // decoded tokens at the head of the batch (where the scheduler puts them) take the kernel that splits
     // their keys (a row of its own in the matrix-core kernel would walk its cache alone); the rest the
@@ -579,8 +610,9 @@ void* attend_prepared(Exec& e, const PagedAttention& t, void* raw, long ldq, lon
   } else if (fast_bf16 && a.max_q == 1 && t.hd % 8 == 0 && t.hd <= 256 && (!t.bias || matrix_sizes)) {
     decode_attention(e, t, raw, ldq, N, a.pos, a.row_req, att);
   } else {
-    RUN(e, gibbs_attention_plain_sink(raw, t.kpages, t.vpages, att, e.p.dtype, a.pos, a.row_req, table, width, t.page_size, t.num_pages,
-                                      N, t.nh, t.nkv, t.hd, t.vd, ldq, ldo, t.scale, t.window, t.slopes, t.bias, t.bias_len, t.sink, a.stream));
+    RUN(e, gibbs_attention_plain_masked(raw, t.kpages, t.vpages, att, e.p.dtype, a.pos, a.row_req, table, width, t.page_size, t.num_pages,
+                                        N, t.nh, t.nkv, t.hd, t.vd, ldq, ldo, t.scale, t.window, t.slopes, t.bias, t.bias_len, t.sink, t.chunk,
+                                        t.softcap, a.stream));
   }
   return att;
 }
@@ -618,6 +650,19 @@ struct AttnBody : Body {
   int keep_mode = 0, keep_key = -1, vt = 0;
   const float* lambda = nullptr;
   bool general_prep = false;
+  // what gibbs_plan_attention_gated sets (on top of the projection options): q and k normed per head with a gain before the
+  // rotation; values that are the keys as projected; values turned by their position and the heads' outputs turned back;
+  // chunks instead of a window; capped scores; a sigmoid gate on the heads' outputs from nh * vd further projected columns
+  const float* prep_q_gain = nullptr;
+  const float* prep_k_gain = nullptr;
+  float prep_eps = 0.f;
+  int prep_norm_dim = 0;
+  int v_from_k = 0;
+  const float* v_inv_freq = nullptr;
+  int v_rot = 0;
+  int chunk = 0;
+  float softcap = 0.f;
+  int gate_off = -1;                  // where the gate's columns start in a projected row (< 0: no gate)
   bool extras() const { return !general_prep && (vd != hd || unit_qk || temp_every > 0 || bias); }
   int cache_group() const override { return group; }
   // the fast kernels know rotations only (or no encoding at all)
@@ -650,7 +695,7 @@ struct AttnBody : Body {
     e.give(att);
   }
   PagedAttention paged() const {
-    return PagedAttention{kpages, vpages, num_pages, page_size, group, nh, nkv, hd, vd, scale, window, slopes, bias, bias_t, bias_len, sink};
+    return PagedAttention{kpages, vpages, num_pages, page_size, group, nh, nkv, hd, vd, scale, window, slopes, bias, bias_t, bias_len, sink, chunk, softcap};
   }
   // q/k norm, rotation and the cache write of the step's rows (a mixer that reads another's cache writes nothing)
   void prepare_rows(Exec& e, void* raw, long ldq) const {
@@ -673,9 +718,9 @@ struct AttnBody : Body {
         }
         keep = it->second;
       }
-      RUN(e, gibbs_qkv_prepare(raw, ldq, owns ? kpages : nullptr, owns ? vpages : nullptr, e.p.dtype, proj_bias, inv_freq, rot, variant, cos_sin,
-                               table_len, keep, keep_mode, vt, lambda, e.a.pos, e.a.row_req, table, width, page_size, num_pages, N, nh, nkv, hd, vd,
-                               e.a.stream));
+      RUN(e, gibbs_qkv_prepare_full(raw, ldq, owns ? kpages : nullptr, owns ? vpages : nullptr, e.p.dtype, proj_bias, inv_freq, rot, variant, cos_sin,
+                                    table_len, keep, keep_mode, vt, lambda, e.a.pos, e.a.row_req, table, width, page_size, num_pages, N, nh, nkv, hd, vd,
+                                    prep_q_gain, prep_k_gain, prep_eps, prep_norm_dim, v_from_k, v_inv_freq, v_rot, e.a.stream));
       return;
     }
     if (extras()) {
@@ -707,13 +752,17 @@ struct AttnBody : Body {
   void* attend(Exec& e, void* raw) const {
     const GibbsStepArgs& a = e.a;
     const int N = a.n_rows, kv = owns ? nkv : 0;
-    const long ldq = (long)(nh + kv) * hd + (long)kv * vd, ldo = (long)nh * vd;
+    const long ldq = general_prep ? qkv.O : (long)(nh + kv) * hd + (long)kv * vd, ldo = (long)nh * vd;
     void* att;
     if (e.bf16_run && a.max_q == 1 && raw_ok()) {
       att = attend_decoded(e, raw);
     } else {
       prepare_rows(e, raw, ldq);
       att = attend_prepared(e, paged(), raw, ldq, ldo);
+      // the heads' outputs turned back by the rows' positions, then times the sigmoid of the gate's columns
+      if (general_prep && (v_inv_freq || gate_off >= 0))
+        RUN(e, gibbs_attention_finish(att, ldo, gate_off >= 0 ? (char*)raw + (long)gate_off * e.esize : nullptr, ldq, vd, e.p.dtype, a.pos, v_inv_freq,
+                                      v_rot, variant, N, nh, vd, vt > 0 ? vt : vd, a.stream));
     }
     return att;
   }
@@ -762,6 +811,66 @@ struct GluBody : Body {
     }
     Pending delta;
     delta.data = e.linear(y, down, N, false, true, true, &delta.parts);
+    e.give(y);
+    return delta;
+  }
+};
+
+// ---- a short causal convolution beside the identity on rows that a mixer is about to read: h <- h + conv(h)
+struct ConvInputBody : Body {
+  const float* taps = nullptr;   // [hidden, K], the last one the current token's
+  int K = 0;
+  float* state = nullptr;        // [slots][K - 1][hidden] float32: the requests' last K - 1 rows
+  long slot_stride = 0;
+  Pending general(Exec& e, void* h) const override {
+    const GibbsStepArgs& a = e.a;
+    const int N = a.n_rows, W = e.p.hidden;
+    Pending out{e.take((long)N * W * e.esize), 1};
+    RUN(e, gibbs_causal_conv(h, W, e.p.dtype, taps, nullptr, state, slot_stride, a.row_req, a.cu, a.slot, out.data, 0, W, N, a.n_req, W, K, 0, 1, 1,
+                             a.max_q == 1, a.stream));
+    return out;
+  }
+};
+
+// ---- state-space mixer (a decayed outer-product state per head, one decay per head and token)
+// One product gives [z: inner | x: inner | B: G D | C: G D | dt: H] of the normed rows (inner = H V, D the state size); x, B and
+// C pass a short causal convolution with bias and silu; dt = softplus(dt + dt_bias); per head, with S [D, V] from zero,
+// S = exp(-exp(A_log) dt) S + B (dt x)';  y = S' C + skip x;  then y silu(z), normed in groups, times a gain, projected back.
+struct SsdBody : Body {
+  Matrix in, out;
+  int H = 0, V = 0, D = 0, G = 0, K = 0, norm_groups = 1;
+  const float* taps = nullptr;       // [inner + 2 G D, K]
+  const float* conv_bias = nullptr;  // [inner + 2 G D] or null
+  const float* dt_bias = nullptr;    // [H]
+  const float* a_log = nullptr;      // [H]
+  const float* skip = nullptr;       // [H]
+  const float* gain = nullptr;       // [inner]
+  float* conv_state = nullptr;       // [slots][K - 1][inner + 2 G D]
+  float* rule_state = nullptr;       // [slots][H][D][V]
+  long slot_stride = 0;
+  float eps = 0.f;
+  Pending general(Exec& e, void* h) const override {
+    const GibbsStepArgs& a = e.a;
+    const int N = a.n_rows, inner = H * V, C = inner + 2 * G * D;
+    char* raw = (char*)e.linear(h, in, N, false, false, false, nullptr);
+    float* xbc = (float*)e.take((long)N * C * 4);
+    RUN(e, gibbs_causal_conv(raw + (long)inner * e.esize, in.O, e.p.dtype, taps, conv_bias, conv_state, slot_stride, a.row_req, a.cu, a.slot, xbc, 1, C,
+                             N, a.n_req, C, K, 1, 0, 1, a.max_q == 1, a.stream));
+    float* decay = (float*)e.take((long)N * H * 4);
+    float* xdt = (float*)e.take((long)N * inner * 4);
+    RUN(e, gibbs_ssd_prep(xbc, C, raw + (long)(inner + C) * e.esize, in.O, e.p.dtype, dt_bias, a_log, decay, xdt, N, H, V, a.stream));
+    float* o = (float*)e.take((long)N * inner * 4);
+    RUN(e, gibbs_ssd_rule(xbc + inner + (long)G * D, xbc + inner, C, xdt, inner, decay, rule_state, slot_stride, a.cu, a.slot, o, a.n_req, H, G, D, V,
+                          a.stream));
+    e.give(decay);
+    e.give(xdt);
+    void* y = e.take((long)N * inner * e.esize);
+    RUN(e, gibbs_gated_group_norm(o, xbc, C, skip, V, raw, in.O, gain, eps, norm_groups, y, e.p.dtype, N, inner, a.stream));
+    e.give(o);
+    e.give(xbc);
+    e.give(raw);
+    Pending delta;
+    delta.data = e.linear(y, out, N, false, true, true, &delta.parts);
     e.give(y);
     return delta;
   }
@@ -969,6 +1078,9 @@ struct MoeBody : Body {
   Matrix shared_gate_up, shared_down;   // the shared expert (w null: none): [2 SF, hidden], [hidden, SF]
   int SF = 0, shared_act = 0;
   const float* shared_gate = nullptr;   // [hidden] float32, or null: the shared expert is added as it is
+  // mode 1: scores by a softmax over all router outputs, the choice by score + router_bias, weights the chosen scores over
+  // their sum; the router's last `identity` outputs are experts without matrices whose result is the row itself
+  int mode = 0, identity = 0;
   Pending general(Exec& e, void* h) const override {
     const int N = e.a.n_rows, W = e.p.hidden, pairs = N * top;
     const int bm = gibbs_moe_tile(pairs, E);
@@ -976,7 +1088,7 @@ struct MoeBody : Body {
     int* chosen = (int*)e.take((long)pairs * 4);
     float* weight = (float*)e.take((long)pairs * 4);
     float* sgate = shared_gate ? (float*)e.take((long)N * 4) : nullptr;
-    RUN(e, gibbs_moe_route(h, W, e.p.dtype, router, router_bias, shared_gate, chosen, weight, sgate, N, W, E, top, e.a.stream));
+    RUN(e, gibbs_moe_route_mode(h, W, e.p.dtype, router, router_bias, shared_gate, chosen, weight, sgate, N, W, E + identity, top, mode, e.a.stream));
     int* sorted = (int*)e.take(cap * 4);
     int* place = (int*)e.take((long)pairs * 4);
     int* tile_expert = (int*)e.take(cap / bm * 4);
@@ -1004,6 +1116,12 @@ struct MoeBody : Body {
     }
     Pending delta{e.take((long)N * W * e.esize), 1};
     e.mix_now();      // (an earlier sum that nothing has taken yet)
+    if (identity > 0) {
+      // (the sum reads the rows themselves for the identity experts: it is taken now, while they are there)
+      RUN(e, gibbs_moe_combine_self(y, place, weight, shared, sgate, h, delta.data, e.p.dtype, N, top, W, e.a.stream));
+      e.give(shared); e.give(y); e.give(place); e.give(weight); e.give(sgate);
+      return delta;
+    }
     e.deferred.delta = delta.data;
     e.deferred.y = y; e.deferred.place = place; e.deferred.weight = weight; e.deferred.shared = shared; e.deferred.gate = sgate;
     e.deferred.top = top;
@@ -1089,6 +1207,13 @@ void Exec::run() {
       case Plan::OP_BODY:
         deltas[op.result] = p.bodies[op.body]->general(*this, rows[op.value]);
         break;
+      case Plan::OP_ROWS: {
+        // a body whose result is read as rows by the next body (a filter on what a mixer reads), not added to the stream
+        Pending made = p.bodies[op.body]->general(*this, rows[op.value]);
+        if (made.parts != 1 && !status) status = gibbs_fail("step: a body whose result is read as rows must give whole rows");
+        rows[op.result] = made.data;
+        break;
+      }
       case Plan::OP_ADD:
         settle(x, pending);
         pending = deltas[op.value];
@@ -1130,6 +1255,24 @@ void Exec::run() {
           give(out);
         }
         mix_now();
+        {
+          // the same boundary for RMS norms in groups: x += norm(delta) and the norm of the new x in one kernel
+          const float *gd = nullptr, *gn = nullptr;
+          float ed = 0.f, en = 0.f;
+          int grd = 0, grn = 0;
+          Pending& dd = deltas[op.value];
+          if (next && pending.parts == 0 && dd.data && p.norms[op.norm]->group_rms(&gd, &ed, &grd) && p.norms[next->norm]->group_rms(&gn, &en, &grn)) {
+            void* out = take((long)N * H * esize);
+            RUN(*this, gibbs_group_rmsnorm(x, dd.data, std::max(dd.parts, 1), (long)N * H, gd, ed, grd, gn, en, grn, out, p.dtype, nullptr, N, H, a.stream));
+            give(dd.data);
+            dd = Pending{};
+            give(mirror);
+            mirror = nullptr;
+            rows[next->result] = out;
+            ++i;
+            break;
+          }
+        }
         // (what is pending stays pending: additions into x commute, and the next norm still takes it on its way)
         if (p.norms[op.norm]->add_normed(*this, x, deltas[op.value])) {
           deltas[op.value] = Pending{};
@@ -1188,6 +1331,7 @@ void Exec::run() {
     void* h = S > 1 ? p.norms[p.tail]->run_streams(*this, x, S, nullptr, a.logit_rows, a.n_logits)
                     : p.norms[p.tail]->run(*this, x, pending, a.logit_rows, a.n_logits);
     linear_into(h, p.head, a.n_logits, true, true, a.logits);   // the head: float32 logits straight into the caller's buffer
+    if (p.logit_softcap > 0.f) RUN(*this, gibbs_softcap_rows(a.logits, (long)a.n_logits * p.vocab, p.logit_softcap, a.stream));
     give(h);
   }
   if (a.settle) settle(x, pending);
@@ -1226,7 +1370,7 @@ int check_args(const Plan* p, const GibbsStepArgs* a, bool whole_step) {
                         op.kind == Plan::OP_REINJECT;
     GIBBS_REQUIRE(p->streams == 1 || !of_one, "step: operation %d works on one residual stream, the plan has %d", i, p->streams);
     GIBBS_REQUIRE(!of_streams || p->streams <= 8, "step: %d residual streams (1 to 8)", p->streams);
-    if (op.kind != Plan::OP_HALF && op.kind != Plan::OP_BODY) continue;
+    if (op.kind != Plan::OP_HALF && op.kind != Plan::OP_BODY && op.kind != Plan::OP_ROWS) continue;
     const int g = p->bodies[op.body]->cache_group();
     GIBBS_REQUIRE(g < 0 || (g < a->n_groups && a->tables && a->tables[g] && a->widths[g] > 0), "step: no block table for cache group %d", g);
   }
@@ -1451,6 +1595,87 @@ GIBBS_EXPORT int gibbs_plan_attention_projection(void* plan, int body, int vd, c
   return 0;
 }
 
+GIBBS_EXPORT int gibbs_plan_attention_gated(void* plan, int body, const float* q_gain, const float* k_gain, float qk_eps, int norm_dim,
+                                            int v_from_k, const float* v_inv_freq, int v_rot, int chunk, float softcap, int gate) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  AttnBody* t = p->has_body(body) ? dynamic_cast<AttnBody*>(p->bodies[body].get()) : nullptr;
+  if (!t || !t->general_prep || !t->owns) { gibbs_fail("plan: body %d is no attention that owns its pages and takes the projection options", body); return -1; }
+  if (((q_gain || k_gain) && !(norm_dim > 0 && norm_dim <= t->hd)) || (v_inv_freq && !(v_rot > 0 && v_rot % 2 == 0 && v_rot <= t->vd)) || chunk < 0 ||
+      (chunk > 0 && t->window > 0) || softcap < 0.f || (v_from_k && (t->keep_mode || v_inv_freq || t->vd > t->hd))) {
+    gibbs_fail("plan: bad options of a gated attention (norm over %d of %d, %d turned value channels of %d, chunks of %d, window %d)", norm_dim, t->hd, v_rot, t->vd, chunk, t->window);
+    return -1;
+  }
+  t->prep_q_gain = q_gain; t->prep_k_gain = k_gain; t->prep_eps = qk_eps; t->prep_norm_dim = norm_dim; t->v_from_k = v_from_k;
+  t->v_inv_freq = v_inv_freq; t->v_rot = v_inv_freq ? v_rot : 0; t->chunk = chunk; t->softcap = softcap;
+  int columns = (t->nh + t->nkv) * t->hd + (v_from_k ? 0 : t->nkv * t->vd);
+  t->gate_off = gate ? columns : -1;
+  if (gate) columns += t->nh * t->vd;
+  t->qkv.O = columns;
+  return 0;
+}
+
+GIBBS_EXPORT int gibbs_plan_norm_group_rms(void* plan, const float* gain, float eps, int groups) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  if (!gain || groups < 1 || p->hidden % groups) { gibbs_fail("plan: an RMS norm in %d parts of a width of %d, or no gain", groups, p->hidden); return -1; }
+  auto n = std::make_unique<GroupRmsNorm>();
+  n->gain = gain; n->eps = eps; n->groups = groups;
+  p->norms.push_back(std::move(n));
+  return (int)p->norms.size() - 1;
+}
+
+GIBBS_EXPORT int gibbs_plan_body_conv_input(void* plan, const float* taps, int K, float* state, long slot_stride) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  if (!(taps && state && K >= 1 && slot_stride >= (long)(K - 1) * p->hidden)) { gibbs_fail("plan: bad input convolution K=%d", K); return -1; }
+  auto b = std::make_unique<ConvInputBody>();
+  b->taps = taps; b->K = K; b->state = state; b->slot_stride = slot_stride;
+  p->bodies.push_back(std::move(b));
+  return (int)p->bodies.size() - 1;
+}
+
+GIBBS_EXPORT int gibbs_plan_body_ssd(void* plan, const GibbsSsdSpec* d) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  if (!d || !(d->w_in && d->w_out && d->taps && d->dt_bias && d->a_log && d->skip && d->gain && d->conv_state && d->rule_state && d->heads > 0 &&
+              d->groups > 0 && d->heads % d->groups == 0 && d->state > 0 && d->state <= 256 && d->vdim > 0 && d->taps_per_channel >= 1 &&
+              d->norm_groups > 0 && (d->heads * d->vdim) % d->norm_groups == 0)) {
+    gibbs_fail("plan: bad state-space mixer");
+    return -1;
+  }
+  const int inner = d->heads * d->vdim, C = inner + 2 * d->groups * d->state;
+  if (d->slot_stride < (long)d->heads * d->state * d->vdim || d->slot_stride < (long)(d->taps_per_channel - 1) * C) {
+    gibbs_fail("plan: a state slot of %ld floats is too small for the state-space mixer", d->slot_stride);
+    return -1;
+  }
+  auto b = std::make_unique<SsdBody>();
+  b->in = Matrix{d->w_in, nullptr, inner + C + d->heads, p->hidden};
+  b->out = Matrix{d->w_out, nullptr, p->hidden, inner};
+  b->H = d->heads; b->V = d->vdim; b->D = d->state; b->G = d->groups; b->K = d->taps_per_channel; b->norm_groups = d->norm_groups;
+  b->taps = d->taps; b->conv_bias = d->conv_bias; b->dt_bias = d->dt_bias; b->a_log = d->a_log; b->skip = d->skip; b->gain = d->gain;
+  b->conv_state = d->conv_state; b->rule_state = d->rule_state; b->slot_stride = d->slot_stride; b->eps = d->eps;
+  p->bodies.push_back(std::move(b));
+  return (int)p->bodies.size() - 1;
+}
+
+GIBBS_EXPORT int gibbs_plan_logit_softcap(void* plan, float cap) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  if (!(cap >= 0.f)) { gibbs_fail("plan: logits capped at %g", cap); return -1; }
+  p->logit_softcap = cap;
+  return 0;
+}
+
+GIBBS_EXPORT int gibbs_plan_moe_scores(void* plan, int body, int mode, int identity) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  MoeBody* m = p->has_body(body) ? dynamic_cast<MoeBody*>(p->bodies[body].get()) : nullptr;
+  if (!m || (mode != 0 && mode != 1) || identity < 0 || m->E + identity > 1024 || m->top > m->E + identity) { gibbs_fail("plan: body %d is no mixture of experts, or bad router options", body); return -1; }
+  m->mode = mode; m->identity = identity;
+  return 0;
+}
+
 GIBBS_EXPORT int gibbs_plan_body_moe(void* plan, const GibbsMoeSpec* d) {
   Plan* p = open_plan(plan);
   if (!p) return -1;
@@ -1553,6 +1778,12 @@ GIBBS_EXPORT int gibbs_plan_op_norm(void* plan, int norm) {
   if (!p) return -1;
   if (!p->has_norm(norm)) { gibbs_fail("plan: no norm %d", norm); return -1; }
   return append(p, Plan::OP_NORM, norm, -1, -1, true);
+}
+GIBBS_EXPORT int gibbs_plan_op_rows(void* plan, int body, int value) {
+  Plan* p = open_plan(plan);
+  if (!p) return -1;
+  if (!p->has_body(body) || !known_value(p, value)) { gibbs_fail("plan: body %d of value %d: no such part or value", body, value); return -1; }
+  return append(p, Plan::OP_ROWS, -1, body, value, true);
 }
 GIBBS_EXPORT int gibbs_plan_op_body(void* plan, int body, int value) {
   Plan* p = open_plan(plan);

@@ -129,6 +129,40 @@ struct GibbsTimeMixSpec {
 };
 int gibbs_plan_body_time_mix(void* plan, const struct GibbsTimeMixSpec* spec);
 
+// An attention body that takes the projection options (gibbs_plan_attention_projection first) may further have: q and k
+// divided per head by their root mean square over the first norm_dim channels and multiplied by a gain [norm_dim], before the
+// rotation; values that are the keys as projected, unnormed and unrotated (v_from_k: the projection has no value rows);
+// values turned by their position over their first v_rot channels (pairs as the rotation's variant says, pair m by
+// pos * v_inv_freq[m]) before they are cached, and every head's output turned back by its row's position; chunks (a row
+// sees the keys of its own stretch of `chunk` positions, counted from 0) instead of a window; scores capped as
+// softcap * tanh(s / softcap); and a gate: nh * vd further projected columns whose sigmoid multiplies the heads' outputs.
+// Projected rows are then [q: nh*hd | k: nkv*hd | v: nkv*vd (unless v_from_k) | gate: nh*vd (if gate)].
+int gibbs_plan_attention_gated(void* plan, int body, const float* q_gain, const float* k_gain, float qk_eps, int norm_dim,
+                               int v_from_k, const float* v_inv_freq, int v_rot, int chunk, float softcap, int gate);
+// RMS norm in `groups` equal consecutive parts of the row (each divided by its own root mean square), times gain [hidden].
+int gibbs_plan_norm_group_rms(void* plan, const float* gain, float eps, int groups);
+// A short causal convolution beside the identity, per channel of the model's width: rows -> rows + conv(rows), taps
+// [hidden, K] (the last one the current token's), the requests' last K - 1 rows in state [slots][K - 1][hidden].
+int gibbs_plan_body_conv_input(void* plan, const float* taps, int K, float* state, long slot_stride);
+// State-space mixer.  w_in [2 inner + 2 groups state + heads, hidden] with inner = heads * vdim, rows [z | x | B | C | dt];
+// taps [inner + 2 groups state, taps_per_channel] and conv_bias over x, B, C; dt_bias, a_log, skip [heads]; gain [inner];
+// the gated read-out is normed in norm_groups parts.  States: conv_state [slots][taps - 1][inner + 2 groups state], rule_state
+// [slots][heads][state][vdim], float32.
+struct GibbsSsdSpec {
+  const void* w_in; const void* w_out;
+  const float* taps; const float* conv_bias; const float* dt_bias; const float* a_log; const float* skip; const float* gain;
+  float* conv_state; float* rule_state; long slot_stride;
+  int heads, vdim, state, groups, taps_per_channel, norm_groups;
+  float eps;
+};
+int gibbs_plan_body_ssd(void* plan, const struct GibbsSsdSpec* spec);
+// logits <- cap * tanh(logits / cap) after the head (0: not capped).
+int gibbs_plan_logit_softcap(void* plan, float cap);
+// A mixture of experts' router: mode 0 as described above; mode 1: scores s = softmax over all router outputs, the `top`
+// largest of s + router_bias are chosen, their weights are their scores s over the sum of those (+ 1e-20).  The router
+// then has experts + identity outputs, the last `identity` of which are experts without matrices that return their input.
+int gibbs_plan_moe_scores(void* plan, int body, int mode, int identity);
+
 // Layer norm with gain and bias (either may be null: 1 and 0).
 int gibbs_plan_norm_layer(void* plan, const float* gain, const float* bias, float eps);
 
@@ -167,6 +201,7 @@ int gibbs_plan_embedding_tables(void* plan, const void* pair_table, int buckets,
 int gibbs_plan_op_half(void* plan, int norm, int body);       // x += body(norm(x)), in fused kernels where it can
 int gibbs_plan_op_norm(void* plan, int norm);                 // -> value: norm(x + what is pending)
 int gibbs_plan_op_body(void* plan, int body, int value);      // -> value: body(normed rows)
+int gibbs_plan_op_rows(void* plan, int body, int value);      // -> value: body(normed rows), read as rows by a later body
 int gibbs_plan_op_add(void* plan, int value);                 // x += delta (lazily: it stays pending for the next norm)
 int gibbs_plan_op_drop(void* plan, int value);                // the value is not read again
 int gibbs_plan_op_norm_delta(void* plan, int norm, int value);   // -> value: norm(a body's delta), the stream untouched

@@ -3,6 +3,6 @@ from .base import (ARRANGEMENTS, CONNECTIONS, Connection, register_connection, F
                    PositionEncoding, Rotation, Runtime, build_block, build_feed_forward, build_mixer, build_norm,
                    build_position, register_arrangement, register_feed_forward, register_mixer, register_norm,
                    register_position)
-from . import attention, block, delta, distance_bias, glu, latent, mlp, moe, norm, rope, shortconv, timemix  # noqa: F401  (registration)
+from . import attention, block, convinput, delta, distance_bias, glu, latent, mlp, moe, norm, rope, shortconv, ssd, timemix  # noqa: F401  (registration)
 from .model import DecoderModel
 from .native import NativePlan

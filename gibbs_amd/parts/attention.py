@@ -20,6 +20,15 @@ denominator without key or value and without the score's scale), `v_head_dim` (v
 own), and `value_mix` = {"key": k, "publish": bool}: the layer that publishes hands its values of the step's rows
 to the later layers of the same key, which cache and use  v <- (1 - lambda) v + lambda v_published  with their
 own lambda (tensor `value_mix`, one number; the publishing layer declares it too and never reads it).
+
+With those options (they share the preparation of the step's rows) go further ones: `qk_norm: "before"` (tensors `q_norm`,
+`k_norm` [head_dim], eps `qk_norm_eps`); `values_from_keys` (no value projection: a position's value is its key as
+projected, before norm and rotation); `value_rotation: {"theta": base}` (values are turned by their position over all of
+their channels, pair m by p * base^(-2m / v_head_dim) in the rotation's pairing, cached so, and every head's output is
+turned back by the query's position); `chunk: n` (a row sees the keys of its own stretch of n positions, counted from
+position 0, instead of a window); `softcap: c` (scores become c tanh(s / c) after the scale); `sink: "zero"` (a sink whose
+number is 0 and not learned: one added to the softmax's denominator); `gate` (tensor `gate_proj` [heads * v_head_dim,
+hidden]: the heads' outputs times sigmoid(W_g h), h the rows that the projections read, before the out-projection).
 """
 from __future__ import annotations
 
@@ -49,12 +58,27 @@ class AttentionMixer(Mixer):
         self.v_head_dim = int(p.get("v_head_dim") or self.head_dim)
         self.q_temperature = p.get("q_temperature")
         self.has_bias, self.has_sink = bool(p.get("bias")), bool(p.get("sink"))
+        self.zero_sink = p.get("sink") == "zero"
         self.value_mix = p.get("value_mix")
+        self.values_from_keys = bool(p.get("values_from_keys"))
+        self.value_rotation = p.get("value_rotation")
+        self.chunk = int(p.get("chunk") or 0)
+        self.softcap = float(p.get("softcap") or 0.0)
+        self.gated = bool(p.get("gate"))
+        self.gated_options = bool(self.values_from_keys or self.value_rotation or self.chunk or self.softcap or self.gated or self.zero_sink)
+        if self.gated_options and (self.source is not None or self.q_temperature is not None or self.qk_norm == "unit"):
+            raise ValueError("values from keys, turned values, chunks, capped scores and a gate go with a mixer that owns its pages and has no unit norm or temperature")
+        if self.chunk and self.window is not None:
+            raise ValueError("an attention sees a window or chunks, not both")
+        if self.values_from_keys and (self.v_head_dim > self.head_dim or self.value_mix is not None or self.value_rotation):
+            raise ValueError("values that are the keys are no larger than they, and neither mixed nor turned")
+        if self.value_rotation and (self.v_head_dim % 2 or self.value_mix is not None):
+            raise ValueError("turned values have an even size and are not mixed")
         if self.value_mix is not None and (self.source is not None or int(self.value_mix["key"]) < 0):
             raise ValueError("value mixing needs a key >= 0 and a mixer that owns its pages")
-        if (self.has_bias or self.has_sink or self.value_mix is not None) and (self.qk_norm is not None or self.q_temperature is not None
+        if (self.has_bias or self.has_sink or self.value_mix is not None) and (self.qk_norm == "unit" or self.q_temperature is not None
                                                                               or self.source is not None):
-            raise ValueError("projection biases, a sink and value mixing go with neither a q/k norm nor a temperature nor another layer's cache")
+            raise ValueError("projection biases, a sink and value mixing go with neither a unit norm nor a temperature nor another layer's cache")
         if self.heads % self.kv_heads:
             raise ValueError(f"{self.heads} heads are not a multiple of {self.kv_heads} kv heads")
         if self.qk_norm not in (None, "before", "unit"):
@@ -100,7 +124,11 @@ class AttentionMixer(Mixer):
         t, H, hd, vd = self.spec.tensors, self.hidden, self.head_dim, self.v_head_dim
         decls = [TensorDecl(t["q_proj"], (self.heads * hd, H))]
         if self.source is None:
-            decls += [TensorDecl(t["k_proj"], (self.kv_heads * hd, H)), TensorDecl(t["v_proj"], (self.kv_heads * vd, H))]
+            decls.append(TensorDecl(t["k_proj"], (self.kv_heads * hd, H)))
+            if not self.values_from_keys:
+                decls.append(TensorDecl(t["v_proj"], (self.kv_heads * vd, H)))
+        if self.gated:
+            decls.append(TensorDecl(t["gate_proj"], (self.heads * vd, H)))
         decls.append(TensorDecl(t["out_proj"], (H, self.heads * vd)))
         if self.qk_norm == "before":
             decls.append(TensorDecl(t["q_norm"], (hd,), FLOAT32, init="gain"))
@@ -110,7 +138,7 @@ class AttentionMixer(Mixer):
             decls += [TensorDecl(t["q_bias"], (self.heads * hd,), FLOAT32, init="bias"),
                       TensorDecl(t["k_bias"], (self.kv_heads * hd,), FLOAT32, init="bias"),
                       TensorDecl(t["v_bias"], (self.kv_heads * vd,), FLOAT32, init="bias")]
-        if self.has_sink:
+        if self.has_sink and not self.zero_sink:
             decls.append(TensorDecl(t["sink"], (self.heads,), FLOAT32, init="bias"))
         if self.value_mix is not None:
             decls.append(TensorDecl(t["value_mix"], (), FLOAT32, init="bias"))
@@ -122,7 +150,7 @@ class AttentionMixer(Mixer):
         """Options that take the preparation of the step's rows with biases, partial rotation and value mixing."""
         rotated_own_values = (self.v_head_dim != self.head_dim and self.qk_norm is None and self.q_temperature is None
                               and self.spec.position is not None and self.spec.position.kind == "rope")
-        return self.has_bias or self.has_sink or self.value_mix is not None or rotated_own_values
+        return self.has_bias or self.has_sink or self.value_mix is not None or rotated_own_values or self.gated_options
 
     def bind(self, weights: WeightStore, rt: Runtime) -> None:
         self.rt = rt
@@ -141,11 +169,15 @@ class AttentionMixer(Mixer):
             w_out = self._pad_heads(w_out, self.heads, self.v_head_dim, pad, rows=False)
         if self.source is None:
             # one product for q, k and v: rows [Wq; Wk; Wv]
-            wk, wv = weights[t["k_proj"]], weights[t["v_proj"]]
+            wk = weights[t["k_proj"]]
+            wv = None if self.values_from_keys else weights[t["v_proj"]]
+            wg = weights[t["gate_proj"]] if self.gated else None
             if self.padded_dim:
                 wk = self._pad_heads(wk, self.kv_heads, self.head_dim, pad, rows=True)
-                wv = self._pad_heads(wv, self.kv_heads, self.v_head_dim, pad, rows=True)
-            self.w_qkv = torch.cat([wq, wk, wv], dim=0).contiguous()
+                wv = None if wv is None else self._pad_heads(wv, self.kv_heads, self.v_head_dim, pad, rows=True)
+                wg = None if wg is None else self._pad_heads(wg, self.heads, self.v_head_dim, pad, rows=True)
+            # (rows [q | k | v, unless the values are the keys | gate])
+            self.w_qkv = torch.cat([w for w in (wq, wk, wv, wg) if w is not None], dim=0).contiguous()
         else:
             self.w_qkv = wq
         self.w_out = w_out.contiguous()
@@ -161,8 +193,14 @@ class AttentionMixer(Mixer):
             self.proj_bias = torch.cat([stored(weights[t["q_bias"]], self.heads, self.head_dim, hd_s),
                                         stored(weights[t["k_bias"]], self.kv_heads, self.head_dim, hd_s),
                                         stored(weights[t["v_bias"]], self.kv_heads, self.v_head_dim, vd_s)]).contiguous()
-        if self.has_sink:
+        if self.zero_sink:
+            self.sinks = torch.zeros(self.heads, dtype=torch.float32, device=rt.device)
+        elif self.has_sink:
             self.sinks = weights[t["sink"]].contiguous()
+        self.v_inv_freq = None
+        if self.value_rotation:
+            from .rope import rope_inv_freq
+            self.v_inv_freq = torch.from_numpy(rope_inv_freq(self.v_head_dim, float(self.value_rotation["theta"]))).to(rt.device)
         if self.value_mix is not None and not self.value_mix.get("publish"):
             self.mix_weight = weights[t["value_mix"]].reshape(1).contiguous()
         self.q_gain = weights[t["q_norm"]] if self.qk_norm == "before" else None
@@ -185,11 +223,12 @@ class AttentionMixer(Mixer):
         return [self.w_qkv, self.w_out]
 
     def product_shapes(self):
-        kv = self.kv_heads * (self.head_dim + self.v_head_dim) if self.source is None else 0
-        return [(self.heads * self.head_dim + kv, self.hidden), (self.hidden, self.heads * self.v_head_dim)]
+        kv = self.kv_heads * (self.head_dim + (0 if self.values_from_keys else self.v_head_dim)) if self.source is None else 0
+        gate = self.heads * self.v_head_dim if self.gated else 0
+        return [(self.heads * self.head_dim + kv + gate, self.hidden), (self.hidden, self.heads * self.v_head_dim)]
 
     def small_tensors(self):
-        own = [t for t in (self.q_gain, self.k_gain, self.slopes, self.proj_bias, self.sinks, self.mix_weight) if t is not None]   # (a score table is the position's)
+        own = [t for t in (self.q_gain, self.k_gain, self.slopes, self.proj_bias, self.sinks, self.mix_weight, self.v_inv_freq) if t is not None]   # (a score table is the position's)
         return own + ([] if self.position is None else list(self.position.small_tensors()))
 
     def fold_input_gain(self, gain: torch.Tensor) -> None:
@@ -223,11 +262,17 @@ class AttentionMixer(Mixer):
             plan.attention_projection(body, v_head_dim=vd, bias=self.proj_bias, sink=self.sinks,
                                       keep_mode=0 if mix is None else (1 if mix.get("publish") else 2),
                                       keep_key=-1 if mix is None else int(mix["key"]), value_dim=self.v_head_dim, weight=self.mix_weight)
+            if self.gated_options or self.qk_norm == "before":
+                plan.attention_gated(body, q_gain=self.q_gain, k_gain=self.k_gain, qk_eps=self.qk_norm_eps, norm_dim=self.head_dim,
+                                     values_from_keys=self.values_from_keys, v_inv_freq=self.v_inv_freq, v_rot=self.v_head_dim,
+                                     chunk=self.chunk, softcap=self.softcap, gate=self.gated)
         return body
 
     def _emit_body(self, plan, cache, hook, head_dim: int) -> int:
+        # (with the projection options the q/k gains travel with them: the body's own are those of the fast paths)
+        prep = self.projection_options()
         return plan.attention(w_qkv=self.w_qkv, p_qkv=self.p_qkv, w_out=self.w_out, p_out=self.p_out, heads=self.heads,
                               kv_heads=self.kv_heads, head_dim=head_dim, scale=self.scale, window=self.window,
-                              q_gain=self.q_gain, k_gain=self.k_gain, qk_eps=self.qk_norm_eps, rotation=self.rot,
+                              q_gain=None if prep else self.q_gain, k_gain=None if prep else self.k_gain, qk_eps=self.qk_norm_eps, rotation=self.rot,
                               kpages=cache.kpages, vpages=cache.vpages, group=cache.group, owns=self.source is None,
                               slopes=self.slopes, rows_hook=hook)

@@ -107,7 +107,9 @@ class SandwichBlock(Block):
 
         x = x + mult * norm1b(mixer(norm1(x)));   x = x + mult * norm2b(ffn(norm2(x)))
 
-    Roles: `norm1`, `mixer`, `norm1b`, and optionally `norm2`, `ffn`, `norm2b` (a layer without a feed-forward).
+    Roles: `norm1`, `mixer`, `norm1b`, and optionally `norm2`, `ffn`, `norm2b` (a layer without a feed-forward), and
+    optionally `mixer_input`: a part with state of its own (kind `conv_input`) through which the mixer reads its normed
+    rows, x = x + mult * norm1b(mixer(mixer_input(norm1(x)))).
     `mult` is the layer spec's `params["residual_mult"]` (default 1); it is multiplied into the gains of the norms
     behind the sublayers when the weights are bound.  The norm of a sublayer's result and its addition into the
     float32 stream are one pass (`plan.add_normed`)."""
@@ -132,11 +134,15 @@ class SandwichBlock(Block):
                 self.ffn.pack_matrices()
 
     def emit(self, plan, caches) -> None:
-        subs = [(self.norm1, lambda: self.mixer.emit(plan, caches["mixer"]), self.norm1b)]
+        subs = [(self.norm1, lambda: self.mixer.emit(plan, caches["mixer"]), self.norm1b, self.named.get("mixer_input"))]
         if self.has_ffn:
-            subs.append((self.norm2, lambda: self.ffn.emit(plan), self.norm2b))
-        for before, body, after in subs:
+            subs.append((self.norm2, lambda: self.ffn.emit(plan), self.norm2b, None))
+        for before, body, after, through in subs:
             h = plan.normed(before.emit(plan))
+            if through is not None:
+                seen = plan.filtered(through.emit(plan, caches["mixer_input"]), h)
+                plan.drop(h)
+                h = seen
             delta = plan.apply(body(), h)
             plan.drop(h)
             plan.add_normed(after.emit(plan), delta)

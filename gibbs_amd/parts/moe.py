@@ -6,6 +6,11 @@ down(act(gate h) * (up h)) without biases; the row's result is the weighted sum 
 `shared` a further expert of its own width runs for every row and is added, times sigmoid(w_gate . h), one number
 per row (`shared: {"inter": F, "activation": .., "gate": bool}`).
 
+`scores: "softmax_all"` is another router: scores s = softmax(z) over all router outputs, the `top` largest of
+s + correction (tensor `correction`, one number per output, seen by the choice alone), weights the chosen experts' s
+divided by their sum (+ 1e-20).  `identity: n`: the router has `experts + n` outputs, and the last n of them are experts
+without matrices whose result is the row itself.  `shared.gate: False` adds the shared expert as it is.
+
 The experts' matrices are kept stacked, [experts, F, hidden] and [experts, hidden, F]: the step sorts its (row,
 choice) pairs by expert on the device and runs the experts' products over tiles of pairs (csrc/moe.hip), so the
 host never learns which experts a step uses."""
@@ -28,13 +33,20 @@ class MoeFeedForward(FeedForward):
         self.experts, self.top, self.inter = int(p["experts"]), int(p["top"]), int(p["inter"])
         self.activation = p.get("activation", "silu")
         self.router_bias_name = spec.tensors.get("router_bias")
+        self.scores = p.get("scores", "softmax_top")
+        self.identity = int(p.get("identity", 0))
+        self.outputs = self.experts + self.identity         # rows of the router
+        if self.scores not in ("softmax_top", "softmax_all") or self.identity < 0:
+            raise ValueError(f"router scores {self.scores!r} ('softmax_top' or 'softmax_all') with {self.identity} identity experts")
+        if self.scores == "softmax_all":
+            self.router_bias_name = spec.tensors.get("correction")
         shared = p.get("shared")
         self.shared_inter = int(shared["inter"]) if shared else 0
         self.shared_activation = (shared or {}).get("activation", self.activation)
         self.shared_gated = bool((shared or {}).get("gate", True))
-        if not 1 <= self.top <= self.experts:
-            raise ValueError(f"{self.top} of {self.experts} experts a token")
-        if self.experts > 1024:
+        if not 1 <= self.top <= self.outputs:
+            raise ValueError(f"{self.top} of {self.outputs} experts a token")
+        if self.outputs > 1024:
             raise ValueError(f"{self.experts} experts are more than the router's kernel takes (1024)")
         for act in (self.activation, self.shared_activation):
             if act not in ops.ACTIVATIONS:
@@ -45,9 +57,9 @@ class MoeFeedForward(FeedForward):
 
     def tensor_decls(self) -> List[TensorDecl]:
         t, H, F = self.spec.tensors, self.hidden, self.inter
-        decls = [TensorDecl(t["router"], (self.experts, H), FLOAT32)]
+        decls = [TensorDecl(t["router"], (self.outputs, H), FLOAT32)]
         if self.router_bias_name is not None:
-            decls.append(TensorDecl(self.router_bias_name, (self.experts,), FLOAT32, init="bias"))
+            decls.append(TensorDecl(self.router_bias_name, (self.outputs,), FLOAT32, init="bias"))
         for e in range(self.experts):
             decls += [TensorDecl(t["gate"][e], (F, H)), TensorDecl(t["up"][e], (F, H)), TensorDecl(t["down"][e], (H, F))]
         if self.shared_inter:
@@ -74,11 +86,12 @@ class MoeFeedForward(FeedForward):
 
     def matrices(self):
         """What a row is multiplied with: the router, its `top` experts (counted as the first ones) and the shared expert."""
-        own = [self.router, self.w_gate[:self.top], self.w_up[:self.top], self.w_down[:self.top]]
+        top = min(self.top, self.experts)
+        own = [self.router, self.w_gate[:top], self.w_up[:top], self.w_down[:top]]
         return own + [m for m in (self.shared_gate_up, self.shared_down) if m is not None]
 
     def product_shapes(self):
-        shapes = [(self.experts, self.hidden)] + [(2 * self.inter, self.hidden), (self.hidden, self.inter)] * self.top
+        shapes = [(self.outputs, self.hidden)] + [(2 * self.inter, self.hidden), (self.hidden, self.inter)] * min(self.top, self.experts)
         if self.shared_inter:
             shapes += [(2 * self.shared_inter, self.hidden), (self.hidden, self.shared_inter)]
         return shapes

@@ -61,6 +61,14 @@ class LatentSpec(ctypes.Structure):
                 ("num_pages", c_int), ("page_size", c_int), ("group", c_int), ("scale", ctypes.c_float), ("eps", ctypes.c_float)]
 
 
+class SsdSpec(ctypes.Structure):
+    """GibbsSsdSpec of csrc/step_plan_api.h."""
+    _fields_ = [("w_in", c_void_p), ("w_out", c_void_p), ("taps", c_void_p), ("conv_bias", c_void_p), ("dt_bias", c_void_p),
+                ("a_log", c_void_p), ("skip", c_void_p), ("gain", c_void_p), ("conv_state", c_void_p), ("rule_state", c_void_p),
+                ("slot_stride", c_long), ("heads", c_int), ("vdim", c_int), ("state", c_int), ("groups", c_int),
+                ("taps_per_channel", c_int), ("norm_groups", c_int), ("eps", ctypes.c_float)]
+
+
 class MoeSpec(ctypes.Structure):
     """GibbsMoeSpec of csrc/step_plan_api.h."""
     _fields_ = [("router", c_void_p), ("router_bias", c_void_p), ("gate", c_void_p), ("up", c_void_p), ("down", c_void_p),
@@ -98,6 +106,13 @@ def declare(lib) -> None:
         "gibbs_plan_body_delta": ([P, POINTER(DeltaSpec)], I),
         "gibbs_plan_body_time_mix": ([P, POINTER(TimeMixSpec)], I),
         "gibbs_plan_norm_layer": ([P, P, P, F], I),
+        "gibbs_plan_norm_group_rms": ([P, P, F, I], I),
+        "gibbs_plan_attention_gated": ([P, I, P, P, F, I, I, P, I, I, F, I], I),
+        "gibbs_plan_body_conv_input": ([P, P, I, P, LG], I),
+        "gibbs_plan_body_ssd": ([P, POINTER(SsdSpec)], I),
+        "gibbs_plan_logit_softcap": ([P, F], I),
+        "gibbs_plan_moe_scores": ([P, I, I, I], I),
+        "gibbs_plan_op_rows": ([P, I, I], I),
         "gibbs_plan_body_latent": ([P, POINTER(LatentSpec)], I),
         "gibbs_plan_body_mlp": ([P, P, P, I, P, F], I),
         "gibbs_plan_streams": ([P, I], I),
@@ -181,6 +196,11 @@ class NativePlan:
     def rms_norm(self, gain: Optional[torch.Tensor], eps: float) -> int:
         (g,) = self._held(gain)
         return self._made(L.library().gibbs_plan_norm_rms(self.handle, g, float(eps)))
+
+    def group_rms_norm(self, gain: torch.Tensor, eps: float, groups: int) -> int:
+        """RMS norm in `groups` equal consecutive parts of the row, the gain over the whole row."""
+        (g,) = self._held(gain)
+        return self._made(L.library().gibbs_plan_norm_group_rms(self.handle, g, float(eps), int(groups)))
 
     def layer_norm(self, gain: Optional[torch.Tensor], bias: Optional[torch.Tensor], eps: float) -> int:
         g, b = self._held(gain, bias)
@@ -278,6 +298,41 @@ class NativePlan:
         self._made(L.library().gibbs_plan_attention_projection(self.handle, int(body), int(v_head_dim), b, s, int(keep_mode),
                                                                int(keep_key), int(value_dim), w))
 
+    def attention_gated(self, body: int, *, q_gain, k_gain, qk_eps: float, norm_dim: int, values_from_keys: bool, v_inv_freq,
+                        v_rot: int, chunk: int, softcap: float, gate: bool) -> None:
+        """Further options of an attention body that takes the projection options: a q/k norm with gains before the
+        rotation, values that are the keys as projected, values turned by their position (and the outputs turned back),
+        chunks instead of a window, capped scores, a sigmoid gate from nh * vd further projected columns."""
+        qg, kg, vf = self._held(q_gain, k_gain, v_inv_freq)
+        self._made(L.library().gibbs_plan_attention_gated(self.handle, int(body), qg, kg, float(qk_eps), int(norm_dim), int(values_from_keys),
+                                                          vf, int(v_rot), int(chunk or 0), float(softcap or 0.0), int(gate)))
+
+    def conv_input(self, *, taps: torch.Tensor, kernel: int, state: torch.Tensor) -> int:
+        """rows -> rows + conv(rows): taps float32 [hidden, kernel], state float32 [slots, kernel - 1, hidden] in the arena."""
+        assert taps.dtype == torch.float32 and taps.is_contiguous() and state.dtype == torch.float32
+        (t,) = self._held(taps)
+        self.keep.append(state)
+        return self._made(L.library().gibbs_plan_body_conv_input(self.handle, t, int(kernel), state.data_ptr(), int(state.stride(0))))
+
+    def ssd(self, m, *, conv_state: torch.Tensor, rule_state: torch.Tensor) -> int:
+        """The state-space mixer `m` (parts/ssd.py) over its states [slots, ...] in the arena."""
+        assert rule_state.dtype == torch.float32 and conv_state.dtype == torch.float32 and rule_state.stride(0) == conv_state.stride(0)
+        d = SsdSpec()
+        d.w_in, d.w_out = self._held(m.w_in, m.w_out)
+        d.taps, d.conv_bias, d.dt_bias, d.a_log, d.skip, d.gain = self._held(m.conv_taps, m.conv_bias, m.dt_bias, m.a_log, m.skip, m.gain)
+        d.conv_state, d.rule_state, d.slot_stride = conv_state.data_ptr(), rule_state.data_ptr(), int(rule_state.stride(0))
+        self.keep += [conv_state, rule_state]
+        d.heads, d.vdim, d.state, d.groups, d.taps_per_channel, d.norm_groups = m.heads, m.vdim, m.state, m.groups, m.taps, m.norm_groups
+        d.eps = m.norm_eps
+        return self._made(L.library().gibbs_plan_body_ssd(self.handle, ctypes.byref(d)))
+
+    def logit_softcap(self, cap: float) -> None:
+        self._made(L.library().gibbs_plan_logit_softcap(self.handle, float(cap)))
+
+    def filtered(self, body: int, value: int) -> int:
+        """-> value: body(normed rows), which a later body reads as its rows (nothing is added to the stream)."""
+        return self._made(L.library().gibbs_plan_op_rows(self.handle, body, value))
+
     def moe(self, m) -> int:
         """The mixture-of-experts feed-forward `m` (parts/moe.py)."""
         from ..ops import ACTIVATIONS
@@ -286,7 +341,10 @@ class NativePlan:
         d.shared_gate_up, d.shared_down, d.shared_gate = self._held(m.shared_gate_up, m.shared_down, m.shared_gate)
         d.experts, d.top, d.F, d.act = m.experts, m.top, m.inter, ACTIVATIONS[m.activation]
         d.shared_F, d.shared_act = m.shared_inter, ACTIVATIONS[m.shared_activation]
-        return self._made(L.library().gibbs_plan_body_moe(self.handle, ctypes.byref(d)))
+        body = self._made(L.library().gibbs_plan_body_moe(self.handle, ctypes.byref(d)))
+        if m.scores == "softmax_all" or m.identity:
+            self._made(L.library().gibbs_plan_moe_scores(self.handle, body, int(m.scores == "softmax_all"), int(m.identity)))
+        return body
 
     def glu_clamped(self, body: int, *, alpha: float, limit: float) -> None:
         self._made(L.library().gibbs_plan_glu_clamped(self.handle, int(body), float(alpha), float(limit)))
@@ -460,6 +518,8 @@ class NativePlan:
                 plan.reinject()
             model.blocks[i].emit(plan, views[run])
         plan.tail(model.final_norm.emit(plan))
+        if model.spec.logit_softcap:
+            plan.logit_softcap(model.spec.logit_softcap)
         return plan
 
     # ------------------------------------------------------------------ running

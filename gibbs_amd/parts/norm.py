@@ -38,6 +38,31 @@ class RMSNorm(Norm):
         return plan.rms_norm(self.gain, self.spec.eps)
 
 
+@register_norm("group_rms")
+class GroupRMSNorm(Norm):
+    """The row in `groups` equal consecutive parts, each divided by its own sqrt(mean(part^2) + eps); then the whole times
+    the gain.  One part is the plain RMS norm (whose kernels and gain folding `"rms"` keeps for itself)."""
+
+    def __init__(self, spec, width):
+        super().__init__(spec, width)
+        self.groups = int(spec.groups)
+        if self.groups < 1 or width % self.groups:
+            raise ValueError(f"a row of {width} values cannot be normed in {self.groups} equal parts")
+
+    def tensor_decls(self) -> List[TensorDecl]:
+        return [TensorDecl(self.spec.weight, (self.width,), FLOAT32, init="gain")]
+
+    def bind(self, weights: WeightStore, rt: Runtime) -> None:
+        self.rt = rt
+        self.gain = weights[self.spec.weight]
+
+    def small_tensors(self):
+        return [self.gain]
+
+    def emit(self, plan) -> int:
+        return plan.group_rms_norm(self.gain, self.spec.eps, self.groups)
+
+
 @register_norm("layer")
 class LayerNorm(Norm):
     def tensor_decls(self) -> List[TensorDecl]:
