@@ -175,6 +175,8 @@ struct DecodeArgs {
   int bias_len;
   // a sink per head, or null: [nh]; the softmax's denominator also holds exp(sink[h]) (natural units, not scaled)
   const float* sink;
+  int chunk;       // > 0: a row sees the keys of its own stretch of `chunk` positions (counted from 0) instead of a window
+  float softcap;   // > 0: scaled scores are capped as softcap * tanh(s / softcap)
 };
 
 // Folds stream b (mb, lb, ab) into stream a.
@@ -233,7 +235,7 @@ __global__ __launch_bounds__(NW * WAVE, GT <= 4 ? (NW == 8 ? 4 : 3) : 2) void at
     pre_page[i] = (a.ids_whole && j < a.n_ids) ? table[j] : 0;
   }
   const int p = a.pos[row];
-  const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
+  const int lo = a.chunk > 0 ? p - p % a.chunk : (a.window > 0 ? max(0, p - a.window + 1) : 0);
   const int len = p + 1 - lo;
   int per = (len + a.n_splits - 1) / a.n_splits;
   constexpr int UNIT = NW * (MM ? TILE : KPW);   // every wave gets whole tiles (or whole steps of keys)
@@ -450,6 +452,13 @@ __global__ __launch_bounds__(NW * WAVE, GT <= 4 ? (NW == 8 ? 4 : 3) : 2) void at
             s4[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qb[s2], s4[c], 0, 0, 0);
           }
         }
+        if (a.softcap > 0.f) {   // (in the raw scores' units: the scale follows)
+          const float cap_raw = a.softcap / a.scale, cap_inv = a.scale / a.softcap;
+#pragma unroll
+          for (int c = 0; c < 2; ++c)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s4[c][i] = cap_raw * tanhf(s4[c][i] * cap_inv);
+        }
         if (a.bias) {
           const float* bias = a.bias + (size_t)(kvh * G + g0 + min(lr, gcount - 1)) * a.bias_len;
 #pragma unroll
@@ -520,6 +529,7 @@ __global__ __launch_bounds__(NW * WAVE, GT <= 4 ? (NW == 8 ? 4 : 3) : 2) void at
   #pragma unroll
           for (int i = 0; i < EPL; ++i) d = fmaf(qf[g][i], kf[i], d);
           d = group_sum<LPK>(d);
+          if (a.softcap > 0.f) d = a.softcap * tanhf(d / a.softcap);   // (q was scaled: these are the scaled scores)
           const float m_new = fmaxf(m[g], d);
           const float keep = __expf(m[g] - m_new);
           const float w = __expf(d - m_new);
@@ -687,7 +697,7 @@ int run_decode(const bf16* q, bf16* kpages, bf16* vpages, bf16* out, float* part
   GIBBS_REQUIRE(!a.bias || (mm_can && kind != 1), "attention_decode: a bias on the scores takes the matrix-core kernel (head sizes in steps of 16 up to 128)");
   const bool mm = kind == 2 || (kind == 0 && mm_can);
   const long ids = (bound + a.page_size - 1) / a.page_size;
-  a.ids_whole = a.window == 0 && ids <= SEG_PAGES;
+  a.ids_whole = a.window == 0 && a.chunk == 0 && ids <= SEG_PAGES;
   a.n_ids = (int)min(ids, (long)a.max_pages);
   if (lanes <= 2) launch_waves<2, RAW>(waves, mm, gt, grid, stream, q, kpages, vpages, partial, out, a);
   else if (lanes <= 4) launch_waves<4, RAW>(waves, mm, gt, grid, stream, q, kpages, vpages, partial, out, a);

@@ -14,11 +14,16 @@ GIBBS_EXPORT long gibbs_attention_decode_workspace(int n_rows, int nh, int hd, i
 // kind: 0 choose, 1 vector units, 2 matrix cores; max_keys: a bound on the keys of any row (0: the block table's width).
 // bias (or null): float32 [nh, bias_len], the score of a key d positions back gets bias[h][min(d, bias_len - 1)] * scale added.
 // sink (or null): float32 [nh], a term exp(sink[h]) in the softmax's denominator that has no key and no value.
-GIBBS_EXPORT int gibbs_attention_decode_sink(const void* q, const void* kpages, const void* vpages, void* out, float* partial,
-                                             const int* pos, const int* row_req, const int* table, int max_pages,
-                                             int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, long ldq,
-                                             long ldo, float scale, int window, int n_splits, int waves, int kind, int max_keys,
-                                             const float* bias, int bias_len, const float* sink, hipStream_t stream) {
+// chunk > 0: a row sees the keys of its own stretch of `chunk` positions, counted from position 0 (no window then).
+// softcap > 0: scores become softcap * tanh(score * scale / softcap) (needs a positive scale).
+GIBBS_EXPORT int gibbs_attention_decode_masked(const void* q, const void* kpages, const void* vpages, void* out, float* partial,
+                                               const int* pos, const int* row_req, const int* table, int max_pages,
+                                               int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, long ldq,
+                                               long ldo, float scale, int window, int n_splits, int waves, int kind, int max_keys,
+                                               const float* bias, int bias_len, const float* sink, int chunk, float softcap,
+                                               hipStream_t stream) {
+  GIBBS_REQUIRE(chunk >= 0 && !(chunk > 0 && window > 0) && softcap >= 0.f && (softcap == 0.f || scale > 0.f),
+                "attention_decode: a window of %d with chunks of %d, or scores capped at %g with a scale of %g", window, chunk, softcap, scale);
   GIBBS_REQUIRE(!bias || (bias_len > 0 && scale > 0.f), "attention_decode: an empty table of score biases, or a scale that is not positive");
   GIBBS_REQUIRE(n_rows >= 0 && nh > 0 && nkv > 0 && hd > 0, "attention_decode: bad sizes rows=%d heads=%d kv=%d hd=%d", n_rows, nh, nkv, hd);
   GIBBS_REQUIRE(nh % nkv == 0, "attention_decode: %d heads are not a multiple of %d kv heads", nh, nkv);
@@ -31,9 +36,18 @@ GIBBS_EXPORT int gibbs_attention_decode_sink(const void* q, const void* kpages, 
   DecodeArgs a{};
   a.pos = pos; a.row_req = row_req; a.table = table; a.max_pages = max_pages; a.page_size = page_size;
   a.num_pages = num_pages; a.nh = nh; a.nkv = nkv; a.hd = hd; a.ldq = ldq; a.ldo = ldo; a.scale = scale;
-  a.window = window; a.n_splits = n_splits; a.bias = bias; a.bias_len = bias_len; a.sink = sink;
+  a.window = window; a.n_splits = n_splits; a.bias = bias; a.bias_len = bias_len; a.sink = sink; a.chunk = chunk; a.softcap = softcap;
   // the kernel only reads the pages here
   return run_decode<false>((const bf16*)q, (bf16*)kpages, (bf16*)vpages, (bf16*)out, partial, a, n_rows, waves, kind, max_keys, stream);
+}
+
+GIBBS_EXPORT int gibbs_attention_decode_sink(const void* q, const void* kpages, const void* vpages, void* out, float* partial,
+                                             const int* pos, const int* row_req, const int* table, int max_pages,
+                                             int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, long ldq,
+                                             long ldo, float scale, int window, int n_splits, int waves, int kind, int max_keys,
+                                             const float* bias, int bias_len, const float* sink, hipStream_t stream) {
+  return gibbs_attention_decode_masked(q, kpages, vpages, out, partial, pos, row_req, table, max_pages, page_size, num_pages, n_rows, nh,
+                                       nkv, hd, ldq, ldo, scale, window, n_splits, waves, kind, max_keys, bias, bias_len, sink, 0, 0.f, stream);
 }
 
 GIBBS_EXPORT int gibbs_attention_decode_bias(const void* q, const void* kpages, const void* vpages, void* out, float* partial,

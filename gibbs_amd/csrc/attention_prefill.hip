@@ -75,6 +75,8 @@ struct PrefillArgs {
   int bias_len;
   // a sink per head, or null: [nh]; the softmax's denominator also holds exp(sink[h]) (natural units, not scaled)
   const float* sink;
+  int chunk;       // > 0: a row sees the keys of its own stretch of `chunk` positions (counted from 0) instead of a window
+  float softcap;   // > 0: scaled scores are capped as softcap * tanh(s / softcap)
 };
 
 // DT: head size = 16 * DT.  POW2: the page size is a power of two (shifts instead of divisions: an
@@ -149,7 +151,7 @@ __global__ __launch_bounds__(256 * HPW) __attribute__((amdgpu_waves_per_eu(DT <=
   }
   // the query row this lane owns in S^T and O^T: wave*16 + lr; it sees keys above lo_row up to pos_row
   const int pos_row = p0 + min(wave * 16 + lr, rows_here - 1);
-  const int lo_row = a.window > 0 ? pos_row - a.window : -1;
+  const int lo_row = a.chunk > 0 ? pos_row - pos_row % a.chunk - 1 : (a.window > 0 ? pos_row - a.window : -1);
 
   // a finite stand-in for 'no key seen yet': exp2 of anything minus it is 0, with no special cases
   float m = -1e30f, l = 0.f;   // maximum of the raw scores; sum of this lane's share of the row
@@ -159,9 +161,11 @@ __global__ __launch_bounds__(256 * HPW) __attribute__((amdgpu_waves_per_eu(DT <=
 
   const float scale2 = a.scale * 1.44269504088896340736f;
   const int last_pos = p0 + rows_here - 1;
-  const int first_key = a.window > 0 ? max(0, p0 - a.window + 1) : 0;
+  const int first_key = a.chunk > 0 ? p0 - p0 % a.chunk : (a.window > 0 ? max(0, p0 - a.window + 1) : 0);
   const int wave_last = p0 + min(wave * 16 + 15, rows_here - 1);
-  const int wave_first_key = a.window > 0 ? max(0, p0 + wave * 16 - a.window + 1) : 0;
+  const int wave_first_key = a.chunk > 0 ? (p0 + wave * 16) - (p0 + wave * 16) % a.chunk : (a.window > 0 ? max(0, p0 + wave * 16 - a.window + 1) : 0);
+  // (capped scores: in the raw scores' units, so that the scale that follows is the same for all)
+  const float cap_raw = a.softcap > 0.f ? a.softcap / a.scale : 0.f, cap_inv = a.softcap > 0.f ? a.scale / a.softcap : 0.f;
 
   // One tile ahead: the next tile's keys and values travel from memory to registers while the
   // matrix cores work on the current tile, and go to LDS once everyone is done with it.
@@ -244,6 +248,12 @@ __global__ __launch_bounds__(256 * HPW) __attribute__((amdgpu_waves_per_eu(DT <=
   auto weights = [&](floatx4 (&s4)[4], int key0, bf16x8 (&pf)[2]) {
     // mask by position (only the tiles on the rows' diagonal, or with a window: the same for the whole wave,
     // and said so, or the selects are done for every tile), row maximum (of the raw scores: the scale is positive)
+    if (a.softcap > 0.f) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s4[c][i] = cap_raw * tanhf(s4[c][i] * cap_inv);
+    }
     if (a.bias) {
       const float* bias = a.bias + (size_t)head * a.bias_len;
 #pragma unroll
@@ -254,7 +264,7 @@ __global__ __launch_bounds__(256 * HPW) __attribute__((amdgpu_waves_per_eu(DT <=
           s4[c][i] += bias[min(max(back, 0), a.bias_len - 1)];
         }
     }
-    const bool need_mask = __builtin_amdgcn_readfirstlane((int)(key0 + BN - 1 > p0 + wave * 16 || a.window > 0)) != 0;
+    const bool need_mask = __builtin_amdgcn_readfirstlane((int)(key0 + BN - 1 > p0 + wave * 16 || a.window > 0 || a.chunk > 0)) != 0;
     if (need_mask) {
 #pragma unroll
       for (int c = 0; c < 4; ++c)
@@ -435,11 +445,16 @@ void launch_prefill(dim3 grid, int heads_per_wg, hipStream_t stream, const bf16*
 // rule for it is gibbs_rule_prefill_heads).
 // bias (or null): float32 [nh, bias_len], the score of a key d positions back gets bias[h][min(d, bias_len - 1)] * scale added.
 // sink (or null): float32 [nh], a term exp(sink[h]) in the softmax's denominator that has no key and no value.
-GIBBS_EXPORT int gibbs_attention_prefill_sink(const void* q, const void* kpages, const void* vpages, void* out, float* partial,
-                                              const int* cu, const int* ctx, const int* table, int n_req, int max_pages,
-                                              int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, long ldq,
-                                              long ldo, float scale, int window, int n_splits, int first_row, int heads_per_wg,
-                                              const float* bias, int bias_len, const float* sink, hipStream_t stream) {
+// chunk > 0: a row sees the keys of its own stretch of `chunk` positions, counted from position 0 (no window then).
+// softcap > 0: scores become softcap * tanh(score * scale / softcap) (needs a positive scale).
+GIBBS_EXPORT int gibbs_attention_prefill_masked(const void* q, const void* kpages, const void* vpages, void* out, float* partial,
+                                                const int* cu, const int* ctx, const int* table, int n_req, int max_pages,
+                                                int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, long ldq,
+                                                long ldo, float scale, int window, int n_splits, int first_row, int heads_per_wg,
+                                                const float* bias, int bias_len, const float* sink, int chunk, float softcap,
+                                                hipStream_t stream) {
+  GIBBS_REQUIRE(chunk >= 0 && !(chunk > 0 && window > 0) && softcap >= 0.f && (softcap == 0.f || scale > 0.f),
+                "attention_prefill: a window of %d with chunks of %d, or scores capped at %g with a scale of %g", window, chunk, softcap, scale);
   GIBBS_REQUIRE(!bias || (bias_len > 0 && scale > 0.f), "attention_prefill: an empty table of score biases, or a scale that is not positive");
   GIBBS_REQUIRE(n_rows >= 0 && n_req >= 0 && nh > 0 && nkv > 0, "attention_prefill: bad sizes rows=%d requests=%d heads=%d kv=%d", n_rows, n_req, nh, nkv);
   GIBBS_REQUIRE(nh % nkv == 0, "attention_prefill: %d heads are not a multiple of %d kv heads", nh, nkv);
@@ -454,7 +469,7 @@ GIBBS_EXPORT int gibbs_attention_prefill_sink(const void* q, const void* kpages,
                 "attention_prefill: %d heads a workgroup (1, 2 or 4 of a kv head's %d; more than one for head sizes up to 64)", heads_per_wg, nh / nkv);
   if (n_rows == 0 || n_req == 0) return 0;
   const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
-  PrefillArgs a{cu, ctx, table, n_req, max_pages, page_size, num_pages, page_shift, nh, nkv, hd, ldq, ldo, scale, window, n_splits, bias, bias_len, sink};
+  PrefillArgs a{cu, ctx, table, n_req, max_pages, page_size, num_pages, page_shift, nh, nkv, hd, ldq, ldo, scale, window, n_splits, bias, bias_len, sink, chunk, softcap};
   dim3 grid(ceil_div(n_rows, BM) + n_req, nh, n_splits);
   const bf16 *qq = (const bf16*)q, *kk = (const bf16*)kpages, *vv = (const bf16*)vpages;
   bf16* oo = (bf16*)out;
@@ -476,6 +491,16 @@ GIBBS_EXPORT int gibbs_attention_prefill_sink(const void* q, const void* kpages,
                            nh, hd, n_splits, ldo, sink);
   }
   GIBBS_LAUNCH_STATUS("attention_prefill");
+}
+
+GIBBS_EXPORT int gibbs_attention_prefill_sink(const void* q, const void* kpages, const void* vpages, void* out, float* partial,
+                                              const int* cu, const int* ctx, const int* table, int n_req, int max_pages,
+                                              int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, long ldq,
+                                              long ldo, float scale, int window, int n_splits, int first_row, int heads_per_wg,
+                                              const float* bias, int bias_len, const float* sink, hipStream_t stream) {
+  return gibbs_attention_prefill_masked(q, kpages, vpages, out, partial, cu, ctx, table, n_req, max_pages, page_size, num_pages, n_rows,
+                                        nh, nkv, hd, ldq, ldo, scale, window, n_splits, first_row, heads_per_wg, bias, bias_len, sink, 0, 0.f,
+                                        stream);
 }
 
 GIBBS_EXPORT int gibbs_attention_prefill_bias(const void* q, const void* kpages, const void* vpages, void* out, float* partial,

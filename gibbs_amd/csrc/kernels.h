@@ -22,6 +22,16 @@ int gibbs_attention_plain_general(const void* q, const void* kpages, const void*
                                   const int* row_req, const int* table, int max_pages, int page_size, int num_pages, int n_rows,
                                   int nh, int nkv, int hd, int vd, long ldq, long ldo, float scale, int window,
                                   const float* slopes, const float* bias, int bias_len, hipStream_t stream);
+int gibbs_attention_prefill_masked(const void* q, const void* kpages, const void* vpages, void* out, float* partial, const int* cu,
+                                   const int* ctx, const int* table, int n_req, int max_pages, int page_size, int num_pages, int n_rows,
+                                   int nh, int nkv, int hd, long ldq, long ldo, float scale, int window, int n_splits, int first_row,
+                                   int heads_per_wg, const float* bias, int bias_len, const float* sink, int chunk, float softcap,
+                                   hipStream_t stream);
+int gibbs_attention_decode_masked(const void* q, const void* kpages, const void* vpages, void* out, float* partial, const int* pos,
+                                  const int* row_req, const int* table, int max_pages, int page_size, int num_pages, int n_rows, int nh,
+                                  int nkv, int hd, long ldq, long ldo, float scale, int window, int n_splits, int waves, int kind,
+                                  int max_keys, const float* bias, int bias_len, const float* sink, int chunk, float softcap,
+                                  hipStream_t stream);
 int gibbs_attention_plain_masked(const void* q, const void* kpages, const void* vpages, void* out, int dtype, const int* pos,
                                  const int* row_req, const int* table, int max_pages, int page_size, int num_pages, int n_rows,
                                  int nh, int nkv, int hd, int vd, long ldq, long ldo, float scale, int window, const float* slopes,

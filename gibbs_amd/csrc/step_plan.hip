@@ -574,11 +574,12 @@ struct PagedAttention {
 };
 void decode_attention(Exec& e, const PagedAttention& t, const void* q, long ldq, int n_rows, const int* pos, const int* row_req, void* o) {
   int n_splits, waves;
-  decode_splits(n_rows, t.nkv, t.nh / t.nkv, e.a.max_seq, t.hd, t.page_size, 0, &n_splits, &waves);
+  // (with chunks a row sees at most a chunk's keys: slices are chosen for that many)
+  decode_splits(n_rows, t.nkv, t.nh / t.nkv, t.chunk > 0 ? std::min(e.a.max_seq, t.chunk) : e.a.max_seq, t.hd, t.page_size, 0, &n_splits, &waves);
   float* partial = n_splits > 1 ? (float*)e.take(gibbs_attention_decode_workspace(n_rows, t.nh, t.hd, n_splits) * 4) : nullptr;
-  RUN(e, gibbs_attention_decode_sink(q, t.kpages, t.vpages, o, partial, pos, row_req, e.table(t.group), e.width(t.group), t.page_size,
-                                     t.num_pages, n_rows, t.nh, t.nkv, t.hd, ldq, (long)t.nh * t.hd, t.scale, t.window, n_splits, waves, 0,
-                                     e.a.max_seq, t.bias_t, t.bias_len, t.sink, e.a.stream));
+  RUN(e, gibbs_attention_decode_masked(q, t.kpages, t.vpages, o, partial, pos, row_req, e.table(t.group), e.width(t.group), t.page_size,
+                                       t.num_pages, n_rows, t.nh, t.nkv, t.hd, ldq, (long)t.nh * t.hd, t.scale, t.window, n_splits, waves, 0,
+                                       e.a.max_seq, t.bias_t, t.bias_len, t.sink, t.chunk, t.softcap, e.a.stream));
   e.give(partial);
 }
 // attention of prepared rows, whatever the step's rows are; returns [N, nh * vd] (row stride ldo)
@@ -592,7 +593,7 @@ void* attend_prepared(Exec& e, const PagedAttention& t, void* raw, long ldq, lon
   // size, and a bias on the scores as a table over the distance (no slopes)
   const bool matrix_sizes = t.hd % 16 == 0 && t.hd <= 128;
   const bool fast_bf16 = e.bf16_run && !t.slopes && t.vd == t.hd && (!t.bias || (t.bias_t && matrix_sizes)) && (!t.sink || t.scale > 0.f) &&
-                         t.chunk == 0 && t.softcap == 0.f;
+                         (t.softcap == 0.f || t.scale > 0.f) && ldq % 8 == 0 && ((uintptr_t)raw % 16) == 0;
   if (fast_bf16 && a.max_q > 1 && matrix_sizes) {
     // decoded tokens at the head of the batch (where the scheduler puts them) take the kernel that splits
     // their keys (a row of its own in the matrix-core kernel would walk its cache alone); the rest the
@@ -600,12 +601,12 @@ void* attend_prepared(Exec& e, const PagedAttention& t, void* raw, long ldq, lon
     const int lead = a.lead_single >= 2 ? a.lead_single : 0;
     if (lead) decode_attention(e, t, raw, ldq, lead, a.pos, a.row_req, att);
     const int rows = N - lead, reqs = a.n_req - lead;
-    const int n_splits = a.max_seq > 0 ? prefill_splits(prefill_tiles(rows, reqs), t.nh, a.max_seq, t.window) : 1;
+    const int n_splits = a.max_seq > 0 ? prefill_splits(prefill_tiles(rows, reqs), t.nh, a.max_seq, t.chunk > 0 ? t.chunk : t.window) : 1;
     float* partial = n_splits > 1 ? (float*)e.take(gibbs_attention_decode_workspace(N, t.nh, t.hd, n_splits) * 4) : nullptr;
-    RUN(e, gibbs_attention_prefill_sink(raw, t.kpages, t.vpages, att, partial, a.cu + lead, a.ctx + lead, table + (long)lead * width, reqs,
-                                        width, t.page_size, t.num_pages, rows, t.nh, t.nkv, t.hd, ldq, ldo, t.scale, t.window, n_splits, lead,
-                                        prefill_heads(rows, reqs, t.nh, t.nkv, t.hd, a.max_seq, n_splits), t.bias_t, t.bias_len, t.sink,
-                                        a.stream));
+    RUN(e, gibbs_attention_prefill_masked(raw, t.kpages, t.vpages, att, partial, a.cu + lead, a.ctx + lead, table + (long)lead * width, reqs,
+                                          width, t.page_size, t.num_pages, rows, t.nh, t.nkv, t.hd, ldq, ldo, t.scale, t.window, n_splits, lead,
+                                          prefill_heads(rows, reqs, t.nh, t.nkv, t.hd, a.max_seq, n_splits), t.bias_t, t.bias_len, t.sink,
+                                          t.chunk, t.softcap, a.stream));
     e.give(partial);
   } else if (fast_bf16 && a.max_q == 1 && t.hd % 8 == 0 && t.hd <= 256 && (!t.bias || matrix_sizes)) {
     decode_attention(e, t, raw, ldq, N, a.pos, a.row_req, att);
@@ -1679,7 +1680,7 @@ GIBBS_EXPORT int gibbs_plan_moe_scores(void* plan, int body, int mode, int ident
 GIBBS_EXPORT int gibbs_plan_body_moe(void* plan, const GibbsMoeSpec* d) {
   Plan* p = open_plan(plan);
   if (!p) return -1;
-  if (!d || !(d->router && d->gate && d->up && d->down && d->experts > 0 && d->experts <= 1024 && d->top > 0 && d->top <= d->experts && d->F > 0 &&
+  if (!d || !(d->router && d->gate && d->up && d->down && d->experts > 0 && d->experts <= 1024 && d->top > 0 && d->top <= 1024 && d->F > 0 &&
               d->act >= 0 && d->act < 4 && (!d->shared_gate_up || (d->shared_down && d->shared_F > 0 && d->shared_act >= 0 && d->shared_act < 4)) &&
               (!d->shared_gate || d->shared_gate_up))) {
     gibbs_fail("plan: bad mixture of experts");

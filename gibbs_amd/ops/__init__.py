@@ -485,8 +485,9 @@ def attention_plain(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kp
                     vpages: torch.Tensor, table: torch.Tensor, n_req: int, pos: torch.Tensor, row_req: torch.Tensor,
                     scale: float, window: Optional[int] = None, out: Optional[torch.Tensor] = None,
                     slopes: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
-                    sink: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Causal grouped-query attention of every row over its request's cache pages.
+                    sink: Optional[torch.Tensor] = None, chunk: int = 0, softcap: float = 0.0) -> torch.Tensor:
+    """Causal grouped-query attention of every row over its request's cache pages (`chunk` > 0: over the keys of the
+    row's own stretch of `chunk` positions counted from 0; `softcap` > 0: scores capped as softcap tanh(s / softcap)).
     q: [N, >= nh*hd] (row stride free); key pages: [num_pages, nkv, page_size, hd]; value pages the same with a
     head size of their own; table: [R, max_pages].
     `slopes` (float32 [nh]): the score of key k for a query at position p gets slopes[h] * (k - p) added.
@@ -505,10 +506,10 @@ def attention_plain(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kp
     if out is None:
         out = torch.empty((n_rows, nh * vd), dtype=q.dtype, device=q.device)
     assert out.shape == (n_rows, nh * vd) and out.dtype == q.dtype and out.is_contiguous()
-    call("gibbs_attention_plain_sink", ptr(q), ptr(kpages), ptr(vpages), ptr(out), dtype_code(q.dtype), ptr(pos),
+    call("gibbs_attention_plain_masked", ptr(q), ptr(kpages), ptr(vpages), ptr(out), dtype_code(q.dtype), ptr(pos),
          ptr(row_req), ptr(table), table.shape[1], page_size, num_pages, n_rows, nh, nkv, hd, vd,
          q.stride(0) if n_rows > 1 else q.shape[1], nh * vd, float(scale), int(window or 0), ptr(slopes), ptr(bias),
-         0 if bias is None else bias.shape[0], ptr(sink), stream())
+         0 if bias is None else bias.shape[0], ptr(sink), int(chunk), float(softcap), stream())
     return out
 
 
@@ -610,7 +611,7 @@ def attention_decode(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, k
                      vpages: torch.Tensor, table: torch.Tensor, n_req: int, pos: torch.Tensor, row_req: Optional[torch.Tensor],
                      scale: float, window: Optional[int] = None, max_seq: int = 0, n_splits: Optional[int] = None,
                      out: Optional[torch.Tensor] = None, waves: Optional[int] = None, kind: str = "auto",
-                     sink: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     sink: Optional[torch.Tensor] = None, chunk: int = 0, softcap: float = 0.0) -> torch.Tensor:
     """bfloat16 paged attention for rows with few queries and long caches (decoded tokens): the
     keys of each (row, kv head) are cut into `n_splits` slices that run as workgroups of their own
     and are merged afterwards.  Same operands and result as `attention_plain`; `row_req` None says that row n is
@@ -641,10 +642,10 @@ def attention_decode(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, k
         out = torch.empty((n_rows, nh * hd), dtype=q.dtype, device=q.device)
     assert out.shape == (n_rows, nh * hd) and out.dtype == q.dtype and out.is_contiguous()
     assert sink is None or (sink.is_cuda and sink.dtype == torch.float32 and sink.shape == (nh,) and sink.is_contiguous())
-    call("gibbs_attention_decode_sink", ptr(q), ptr(kpages), ptr(vpages), ptr(out), ptr(partial), ptr(pos), ptr(row_req),
+    call("gibbs_attention_decode_masked", ptr(q), ptr(kpages), ptr(vpages), ptr(out), ptr(partial), ptr(pos), ptr(row_req),
          ptr(table), table.shape[1], page_size, num_pages, n_rows, nh, nkv, hd,
          q.stride(0) if n_rows > 1 else q.shape[1], nh * hd, float(scale), int(window or 0), n_splits, int(waves), DECODE_KINDS[kind],
-         int(max_seq), None, 0, ptr(sink), stream())
+         int(max_seq), None, 0, ptr(sink), int(chunk), float(softcap), stream())
     return out
 
 
@@ -658,7 +659,7 @@ def attention_prefill(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, 
                       scale: float, window: Optional[int] = None, out: Optional[torch.Tensor] = None,
                       max_seq: int = 0, n_splits: Optional[int] = None, first_req: int = 0,
                       first_row: int = 0, heads_per_wg: Optional[int] = None,
-                      sink: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      sink: Optional[torch.Tensor] = None, chunk: int = 0, softcap: float = 0.0) -> torch.Tensor:
     """bfloat16 paged causal attention for prompt portions on the matrix cores: rows cu[r] .. cu[r+1]
     of request r sit at positions ctx[r] ..; same result as `attention_plain`.  Head sizes: multiples
     of 16 up to 128.  `max_seq`: a bound on the keys of any row, from which the number of key slices
@@ -688,10 +689,10 @@ def attention_prefill(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, 
     if n_splits > 1:
         partial = torch.empty(slices_workspace(n_rows, nh, hd, n_splits), dtype=torch.float32, device=q.device)
     assert sink is None or (sink.is_cuda and sink.dtype == torch.float32 and sink.shape == (nh,) and sink.is_contiguous())
-    call("gibbs_attention_prefill_sink", ptr(q), ptr(kpages), ptr(vpages), ptr(out), ptr(partial), ptr(cu[first_req:]),
+    call("gibbs_attention_prefill_masked", ptr(q), ptr(kpages), ptr(vpages), ptr(out), ptr(partial), ptr(cu[first_req:]),
          ptr(ctx[first_req:]), ptr(table[first_req:]), reqs, table.shape[1], page_size, num_pages, rows, nh, nkv, hd,
          q.stride(0) if n_rows > 1 else q.shape[1], nh * hd, float(scale), int(window or 0), int(n_splits), int(first_row),
-         int(heads_per_wg), None, 0, ptr(sink), stream())
+         int(heads_per_wg), None, 0, ptr(sink), int(chunk), float(softcap), stream())
     return out
 
 

@@ -66,6 +66,33 @@ _SIGNATURES = {
     "gibbs_attention_decode_sink": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                     c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_int,
                                     c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p],
+    "gibbs_attention_plain_masked": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                                     c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_void_p,
+                                     c_void_p, c_int, c_void_p, c_int, c_float, c_void_p],
+    "gibbs_attention_prefill_masked": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                       c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_int, c_int, c_int,
+                                       c_void_p, c_int, c_void_p, c_int, c_float, c_void_p],
+    "gibbs_attention_decode_masked": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                      c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_int,
+                                      c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_float, c_void_p],
+    "gibbs_qkv_prepare_full": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_int,
+                               c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                               c_void_p, c_void_p, c_float, c_int, c_int, c_void_p, c_int, c_void_p],
+    "gibbs_attention_finish": [c_void_p, c_long, c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                               c_void_p],
+    "gibbs_group_rmsnorm": [c_void_p, c_void_p, c_int, c_long, c_void_p, c_float, c_int, c_void_p, c_float, c_int, c_void_p, c_int, c_void_p,
+                            c_int, c_int, c_void_p],
+    "gibbs_gated_group_norm": [c_void_p, c_void_p, c_long, c_void_p, c_int, c_void_p, c_long, c_void_p, c_float, c_int, c_void_p, c_int, c_int,
+                               c_int, c_void_p],
+    "gibbs_causal_conv": [c_void_p, c_long, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_long,
+                          c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "gibbs_ssd_prep": [c_void_p, c_long, c_void_p, c_long, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "gibbs_ssd_rule": [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                       c_int, c_int, c_int, c_void_p],
+    "gibbs_moe_route_mode": [c_void_p, c_long, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                             c_int, c_void_p],
+    "gibbs_moe_combine_self": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "gibbs_softcap_rows": [c_void_p, c_long, c_float, c_void_p],
     "gibbs_embed_tables": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_long,
                            c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gibbs_store_last_token": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_int, c_void_p],

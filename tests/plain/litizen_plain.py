@@ -119,13 +119,15 @@ def window_attention_mixer(h, w, p: str, m: dict, positions, eps: float) -> np.n
     q = (h @ w[p + "q"].T).reshape(T, H, D)
     k = (h @ w[p + "k"].T).reshape(T, G, D)
     v = k.copy()
-    q = group_rms_norm(q, w[p + "q.norm"], eps, 1)
-    k = group_rms_norm(k, w[p + "k.norm"], eps, 1)
+    if p + "q.norm" in w:
+        q = group_rms_norm(q, w[p + "q.norm"], eps, 1)
+        k = group_rms_norm(k, w[p + "k.norm"], eps, 1)
     rot = m.get("rot")
-    if rot is not None and int(rot["dims"]) > 0:
+    if rot is not None and int(rot.get("dims", 0)) > 0:
         q = rotate(q, positions, float(rot["base"]), int(rot["dims"]))
         k = rotate(k, positions, float(rot["base"]), int(rot["dims"]))
-    o = masked_attention(q, k, v, float(m["scale"]), visible_window(T, int(m["mask"]["size"])), sink=np.zeros(H, dtype=F64))
+    size = (m.get("mask") or {}).get("size")
+    o = masked_attention(q, k, v, float(m["scale"]), visible_window(T, T if size is None else int(size)), sink=np.zeros(H, dtype=F64))
     o = o.reshape(T, H * V) * sigmoid(h @ w[p + "g"].T)
     return o @ w[p + "o"].T
 
@@ -140,11 +142,12 @@ def chunk_attention_mixer(h, w, p: str, m: dict, positions) -> np.ndarray:
     v = (h @ w[p + "v"].T).reshape(T, G, V)
     rot = m["rot"]
     base = float(rot["base"])
-    if int(rot["dims"]) > 0:
+    if int(rot.get("dims", 0)) > 0:
         q = rotate(q, positions, base, int(rot["dims"]))
         k = rotate(k, positions, base, int(rot["dims"]))
     v = rotate(v, positions, base, V)
-    o = masked_attention(q, k, v, float(m["scale"]), visible_chunk(T, int(m["mask"]["size"])), sink=w[p + "sink"],
+    size = (m.get("mask") or {}).get("size")
+    o = masked_attention(q, k, v, float(m["scale"]), visible_chunk(T, T if size is None else int(size)), sink=w.get(p + "sink"),
                          softcap=m.get("softcap"))
     o = rotate(o, positions, base, V, sign=-1.0)
     o = o.reshape(T, H * V) * sigmoid(h @ w[p + "g"].T)
@@ -202,10 +205,23 @@ def route(h, router, correction, top: int):
     return chosen, picked / (picked.sum(-1, keepdims=True) + 1e-20)
 
 
-def moe_ff(h, w, p: str, mlp: dict) -> np.ndarray:
+def route_margin(h, router, correction, top: int) -> np.ndarray:
+    """Per row, how far the last chosen expert's score + correction lies above the best one that was not chosen (inf
+    where every expert is chosen): a choice closer than the rounding of h may fall the other way in another precision."""
+    z = h @ router.T
+    z = z - z.max(-1, keepdims=True)
+    s = np.exp(z)
+    s = np.sort(s / s.sum(-1, keepdims=True) + correction[None, :], axis=-1)[:, ::-1]
+    return s[:, top - 1] - s[:, top] if top < s.shape[1] else np.full(h.shape[0], np.inf)
+
+
+def moe_ff(h, w, p: str, mlp: dict, margins_out=None) -> np.ndarray:
     """Experts 0 .. E-1 are gated feed-forwards; the last `identity` router outputs are experts that return their input."""
     E, top = int(mlp["router"]["experts"]), int(mlp["router"]["top"])
-    chosen, weights = route(h, w[p + "router"], w[p + "correction"], top)
+    correction = w.get(p + "correction", np.zeros(w[p + "router"].shape[0]))
+    chosen, weights = route(h, w[p + "router"], correction, top)
+    if margins_out is not None:
+        margins_out.append(route_margin(h, w[p + "router"], correction, top))
     out = np.zeros_like(h, dtype=F64)
     for t in range(h.shape[0]):
         for e, wt in zip(chosen[t], weights[t]):
@@ -219,15 +235,16 @@ def moe_ff(h, w, p: str, mlp: dict) -> np.ndarray:
     return out
 
 
-def feed_forward(h, w, p: str, mlp: dict) -> np.ndarray:
+def feed_forward(h, w, p: str, mlp: dict, margins_out=None) -> np.ndarray:
     if mlp["kind"] == "dense":
         return gated_ff(h, w[p + "gate"], w[p + "up"], w[p + "down"])
-    return moe_ff(h, w, p, mlp)
+    return moe_ff(h, w, p, mlp, margins_out)
 
 
 # --------------------------------------------------------------------------- the model
-def forward(cfg: dict, weights: dict, tokens, return_layers: bool = False):
-    """Logits [T, vocab] of one sequence (and the residual stream after every layer, [layers, T, W])."""
+def forward(cfg: dict, weights: dict, tokens, return_layers: bool = False, margins_out=None):
+    """Logits [T, vocab] of one sequence (and the residual stream after every layer, [layers, T, W]).  `margins_out`: a list
+    that receives every expert layer's `route_margin` per token."""
     w = {k: np.asarray(v, dtype=F64) for k, v in weights.items()}
     eps, groups = float(cfg["norm"]["eps"]), int(cfg["norm"].get("groups", 1))
     T = len(tokens)
@@ -237,7 +254,9 @@ def forward(cfg: dict, weights: dict, tokens, return_layers: bool = False):
     after = []
     for i, layer in enumerate(cfg["layers"]):
         p, m = f"l{i}.", layer["mixer"]
-        h = input_conv(norm(x, p + "norm1"), w[p + "canon1"])
+        h = norm(x, p + "norm1")
+        if p + "canon1" in w:
+            h = input_conv(h, w[p + "canon1"])
         if layer["type"] == "attention":
             d = window_attention_mixer(h, w, p + "mix.", m, positions, eps)
         elif layer["type"] == "attention_2":
@@ -248,9 +267,9 @@ def forward(cfg: dict, weights: dict, tokens, return_layers: bool = False):
             raise ValueError(layer["type"])
         x = x + norm(d, p + "norm1b")
         if layer.get("mlp") is not None:
-            x = x + norm(feed_forward(norm(x, p + "norm2"), w, p + "mlp.", layer["mlp"]), p + "norm2b")
+            x = x + norm(feed_forward(norm(x, p + "norm2"), w, p + "mlp.", layer["mlp"], margins_out), p + "norm2b")
         after.append(x.copy())
-    logits = norm(x, "final.norm") @ w["head"].T
+    logits = norm(x, "final.norm") @ w["head" if "head" in w else "embed"].T
     cap = cfg.get("logit_softcap")
     if cap:
         logits = cap * np.tanh(logits / cap)
