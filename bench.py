@@ -339,8 +339,31 @@ def ruzinex_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
             "layers": [{"type": "attention", "mixer": mixer, "mlp": mlps[i % 2]} for i in range(layers)]}
 
 
-BESIDE = {"zokepel": ("Zokepel", zokepel_shape, lfm2_shape), "rukosun": ("Rukosun", rukosun_shape, lfm2_attention_shape),
-          "ruzinex": ("Ruzinex", ruzinex_shape, lfm2_attention_shape)}
+def litizen_shape(width: int, ff: int, layers: int, vocab: int) -> dict:
+    """A Litizen model of `layers` layers (state-space, windowed attention, chunked attention in turn) whose sizes resemble a
+    real model's at this width: attention heads of 64 in groups of four, half of every head rotated, a window of 1,024 and
+    chunks of 1,024; a state-space layer of twice the width in heads of 64 with a state of 128 in eight groups; norms in
+    eight parts; four taps in front of every mixer; dense feed-forwards and mixtures of experts in turn, a mixture being
+    16 experts of an eighth of the dense width and 2 identity experts, of which a token takes 4, beside a shared expert of
+    half the dense width."""
+    heads = width // 64
+    kinds = [
+        {"type": "mamba2", "mixer": {"heads": 2 * heads, "vdim": 64, "state": 128, "groups": 8 if (2 * heads) % 8 == 0 else 1, "conv": 4, "norm_groups": 8}},
+        {"type": "attention", "mixer": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 64, "vdim": 64, "scale": 0.125, "mask": {"size": 1024},
+                                        "rot": {"base": 1000000.0, "dims": 32}}},
+        {"type": "attention_2", "mixer": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 64, "vdim": 64, "scale": 0.125, "mask": {"size": 1024},
+                                          "rot": {"base": 10000.0, "dims": 32}, "softcap": 50.0}},
+    ]
+    mlps = [{"kind": "dense", "ff": ff},
+            {"kind": "moe", "expert": {"ff": ff // 8}, "router": {"experts": 16, "identity": 2, "top": 4}, "shared": {"ff": ff // 2}}]
+    return {"architecture": "Litizen", "vocab": vocab, "width": width, "norm": {"eps": 1e-6, "groups": 8}, "canon": {"taps": 4},
+            "embedding": {"scale": 1.0}, "logit_softcap": 30.0,
+            "layers": [dict(kinds[i % 3], mlp=mlps[i % 2]) for i in range(layers)]}
+
+
+# design -> (its name, its shape, the closest model the framework had, that model's shape at equal sizes)
+BESIDE = {"zokepel": ("Zokepel", zokepel_shape, "LFM2", lfm2_shape), "rukosun": ("Rukosun", rukosun_shape, "LFM2", lfm2_attention_shape),
+          "ruzinex": ("Ruzinex", ruzinex_shape, "LFM2", lfm2_attention_shape), "litizen": ("Litizen", litizen_shape, "Ruzinex", ruzinex_shape)}
 
 
 def engine_of(shape: dict, dtype: str, max_requests: int, context: int):
@@ -358,7 +381,7 @@ def engine_of(shape: dict, dtype: str, max_requests: int, context: int):
 
 
 def compare_designs(args) -> int:
-    """`--design zokepel` / `rukosun` / `ruzinex`: prefill and decode speed of that design at a few sizes beside LFM2 at equal
+    """`--design zokepel` / `rukosun` / `ruzinex` / `litizen`: prefill and decode speed of that design at a few sizes beside LFM2 (Litizen: beside Ruzinex) at equal
     width, depth, feed-forward and vocabulary (random weights), with the kernels that each one's time goes to.  One
     JSON line."""
     import faulthandler
@@ -386,9 +409,9 @@ def compare_designs(args) -> int:
     sizes = {"small": [(1024, 4096, 6, 32768)], "medium": [(2048, 8192, 6, 65536)],
              "all": [(1024, 4096, 6, 32768), (2048, 8192, 6, 65536), (4096, 12288, 3, 65536)]}[args.sizes]
     rows = []
-    name, its_shape, lfm2_beside = BESIDE[args.design]
+    name, its_shape, other, other_shape = BESIDE[args.design]
     for width, ff, layers, vocab in sizes:
-        for design, shape in ((name, its_shape(width, ff, layers, vocab)), ("LFM2", lfm2_beside(width, ff, layers, vocab))):
+        for design, shape in ((name, its_shape(width, ff, layers, vocab)), (other, other_shape(width, ff, layers, vocab))):
             print(f"[bench] {design} width {width}: building", file=sys.stderr, flush=True)
             engine = engine_of(shape, args.dtype, max_requests=args.batch, context=4096)
             row = {"design": design, "width": width, "ff": ff, "layers": layers, "vocab": vocab}
@@ -420,9 +443,10 @@ def compare_designs(args) -> int:
 
 def main() -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", choices=["lfm2", "zokepel", "rukosun", "ruzinex"], default="lfm2",
-                    help="zokepel, rukosun, ruzinex: that design beside LFM2 at equal sizes instead of the headline workload")
-    ap.add_argument("--sizes", choices=["small", "medium", "all"], default="medium", help="sizes of --design zokepel / rukosun / ruzinex")
+    ap.add_argument("--design", choices=["lfm2", "zokepel", "rukosun", "ruzinex", "litizen"], default="lfm2",
+                    help="zokepel, rukosun, ruzinex: that design beside LFM2 at equal sizes instead of the headline workload; "
+                         "litizen: beside Ruzinex, the closest design the framework had")
+    ap.add_argument("--sizes", choices=["small", "medium", "all"], default="medium", help="sizes of --design zokepel / rukosun / ruzinex / litizen")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
