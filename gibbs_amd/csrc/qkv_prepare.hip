@@ -51,12 +51,14 @@ struct QkvPrepareArgs {
   int v_rot;
 };
 
-template <typename T>
+// LPH lanes share a head (16 for heads of up to 128 channels: four heads a wave; else the whole wave).
+template <typename T, int LPH>
 __global__ __launch_bounds__(256) void qkv_prepare_kernel(T* __restrict__ rows, T* __restrict__ kpages, T* __restrict__ vpages,
                                                           T* __restrict__ keep, QkvPrepareArgs a) {
+  constexpr int WAVE = LPH;      // (below, "the wave" is the group of lanes that shares a head)
   const int n = blockIdx.x;
-  const int hs = blockIdx.y * (blockDim.x / WAVE) + threadIdx.x / WAVE;
-  const int lane = threadIdx.x % WAVE;
+  const int hs = blockIdx.y * (blockDim.x / LPH) + threadIdx.x / LPH;
+  const int lane = threadIdx.x % LPH;
   if (hs >= a.nh + (a.v_from_k ? 1 : 2) * a.nkv) return;
   const bool is_q = hs < a.nh, is_k = !is_q && hs < a.nh + a.nkv;
   const int g = is_q ? hs : (is_k ? hs - a.nh : hs - a.nh - a.nkv);
@@ -105,7 +107,7 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(T* __restrict__ rows, 
   if (gain) {
     float ss = 0.f;
     for (int e = lane; e < a.norm_dim; e += WAVE) { const float x = raw_value(e); ss = fmaf(x, x, ss); }
-    inv = 1.0f / sqrtf(wave_sum(ss) / (float)a.norm_dim + a.qk_eps);
+    inv = 1.0f / sqrtf((LPH == 64 ? wave_sum(ss) : group_sum<LPH>(ss)) / (float)a.norm_dim + a.qk_eps);
   }
   auto value = [&](int e) -> float { return gain ? (e < a.norm_dim ? raw_value(e) * inv * gain[e] : 0.f) : raw_value(e); };
   if (!is_q && !is_k) {
@@ -302,13 +304,16 @@ GIBBS_EXPORT int gibbs_qkv_prepare_full(void* rows, long ld, void* kpages, void*
       GIBBS_LAUNCH_STATUS("qkv_prepare");
     }
   }
-  const int per_block = 4;
+  const bool narrow = hd <= 128 && vd <= 128;      // four heads a wave
+  const int per_block = narrow ? 16 : 4;
   const dim3 grid(n_rows, ceil_div(nh + 2 * nkv, per_block));
-  if (dtype == GIBBS_F32)
-    qkv_prepare_kernel<float><<<grid, per_block * WAVE, 0, stream>>>((float*)rows, (float*)kpages, (float*)vpages, (float*)keep, a);
-  else if (dtype == GIBBS_BF16)
-    qkv_prepare_kernel<bf16><<<grid, per_block * WAVE, 0, stream>>>((bf16*)rows, (bf16*)kpages, (bf16*)vpages, (bf16*)keep, a);
-  else
+  if (dtype == GIBBS_F32) {
+    if (narrow) qkv_prepare_kernel<float, 16><<<grid, 256, 0, stream>>>((float*)rows, (float*)kpages, (float*)vpages, (float*)keep, a);
+    else qkv_prepare_kernel<float, 64><<<grid, 256, 0, stream>>>((float*)rows, (float*)kpages, (float*)vpages, (float*)keep, a);
+  } else if (dtype == GIBBS_BF16) {
+    if (narrow) qkv_prepare_kernel<bf16, 16><<<grid, 256, 0, stream>>>((bf16*)rows, (bf16*)kpages, (bf16*)vpages, (bf16*)keep, a);
+    else qkv_prepare_kernel<bf16, 64><<<grid, 256, 0, stream>>>((bf16*)rows, (bf16*)kpages, (bf16*)vpages, (bf16*)keep, a);
+  } else
     return gibbs_fail("qkv_prepare: unknown dtype %d", dtype);
   GIBBS_LAUNCH_STATUS("qkv_prepare");
 }

@@ -48,6 +48,66 @@ __global__ void causal_conv_silu_kernel(const T* __restrict__ in, long ld, const
   out[(size_t)n * ld_out + c] = from_float<TO>(acc);
 }
 
+// The same for bfloat16 inputs whose channels come in whole groups of 8: a thread takes 8 neighbouring channels of a row with
+// 16-byte loads.  A workgroup is 64 lanes of channels by CONV_ROWS rows; the taps of its 512 channels, one contiguous stretch of
+// the [C, K] table, come into LDS once (each thread's 8 K taps a word further along, so that the lanes read different banks)
+// instead of as 8 K scattered words per thread.  Sums in ascending j, as above.
+constexpr int CONV_ROWS = 4, CONV_LANES = 64;
+template <typename TO>
+__global__ __launch_bounds__(CONV_ROWS * CONV_LANES) void causal_conv_vec8_kernel(
+    const bf16* __restrict__ in, long ld, const float* __restrict__ taps, const float* __restrict__ bias, float* __restrict__ state,
+    long slot_stride, const int* __restrict__ row_req, const int* __restrict__ cu, const int* __restrict__ slot, TO* __restrict__ out,
+    long ld_out, int n_rows, int C, int K, int shift_state, int act, int residual) {
+  extern __shared__ float s_taps[];    // [CONV_LANES][8 K + 1]
+  const int c0 = blockIdx.y * CONV_LANES * 8;
+  const int span = min(CONV_LANES * 8, C - c0) * K;      // taps of this workgroup's channels
+  const int tid = threadIdx.y * CONV_LANES + threadIdx.x;
+  for (int i = tid; i < span; i += CONV_ROWS * CONV_LANES) s_taps[i + i / (8 * K)] = taps[(size_t)c0 * K + i];
+  __syncthreads();
+  const int n = blockIdx.x * CONV_ROWS + threadIdx.y;
+  const int c = c0 + threadIdx.x * 8;
+  if (n >= n_rows || c >= C) return;
+  const float* tp = s_taps + threadIdx.x * (8 * K + 1);
+  const int r = row_req[n], first = cu[r], t = n - first;
+  float* st = state + (size_t)slot[r] * slot_stride;
+  float acc[8] = {}, own[8] = {};
+  for (int j = 0; j < K; ++j) {
+    const int tt = t - (K - 1) + j;
+    float xv[8];
+    if (tt >= 0) {
+      unpack8(*(const uint4*)(in + (size_t)(first + tt) * ld + c), xv);
+    } else {
+      const float4 a = *(const float4*)(st + (size_t)(K - 1 + tt) * C + c), b = *(const float4*)(st + (size_t)(K - 1 + tt) * C + c + 4);
+      xv[0] = a.x; xv[1] = a.y; xv[2] = a.z; xv[3] = a.w; xv[4] = b.x; xv[5] = b.y; xv[6] = b.z; xv[7] = b.w;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      acc[i] = fmaf(tp[i * K + j], xv[i], acc[i]);
+      own[i] = xv[i];
+    }
+    if (shift_state && j >= 1) {
+      *(float4*)(st + (size_t)(j - 1) * C + c) = make_float4(xv[0], xv[1], xv[2], xv[3]);
+      *(float4*)(st + (size_t)(j - 1) * C + c + 4) = make_float4(xv[4], xv[5], xv[6], xv[7]);
+    }
+  }
+  if (bias) {
+    const float4 b0 = *(const float4*)(bias + c), b1 = *(const float4*)(bias + c + 4);
+    acc[0] += b0.x; acc[1] += b0.y; acc[2] += b0.z; acc[3] += b0.w; acc[4] += b1.x; acc[5] += b1.y; acc[6] += b1.z; acc[7] += b1.w;
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    if (act == CONV_ACT_SILU) acc[i] = acc[i] * sigmoid_f(acc[i]);
+    if (residual) acc[i] += own[i];
+  }
+  TO* o = out + (size_t)n * ld_out + c;
+  if constexpr (sizeof(TO) == 2) {
+    *(uint4*)o = pack8(acc);
+  } else {
+    *(float4*)o = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    *(float4*)(o + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
+  }
+}
+
 // The state after the step: the last K-1 inputs of the request (what the step brought, and before that what
 // the state held).  One thread per (request, channel), entries in ascending order: entry i reads entry
 // i + rows of the old state, which has not been written yet.
@@ -406,7 +466,14 @@ GIBBS_EXPORT int gibbs_causal_conv(const void* in, long ld, int dtype, const flo
                 "causal_conv: bad operands rows=%d requests=%d C=%d K=%d", n_rows, n_req, C, K);
   const dim3 rows(n_rows, ceil_div(C, 256)), reqs(n_req, ceil_div(C, 256));
 #define CONV_ARGS taps, bias, state, slot_stride, row_req, cu, slot
-  if (out_f32 || dtype == GIBBS_F32)
+  const bool vec8 = dtype == GIBBS_BF16 && C % 8 == 0 && ld % 8 == 0 && ((uintptr_t)in % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
+                    ld_out % (out_f32 ? 4 : 8) == 0 && slot_stride % 4 == 0 && ((uintptr_t)state % 16) == 0 && ((uintptr_t)bias % 16) == 0 && K <= 16;
+  if (vec8) {
+    const dim3 grid(ceil_div(n_rows, CONV_ROWS), ceil_div(C, CONV_LANES * 8)), block(CONV_LANES, CONV_ROWS);
+    const size_t lds = (size_t)CONV_LANES * (8 * K + 1) * sizeof(float);
+    if (out_f32) causal_conv_vec8_kernel<float><<<grid, block, lds, stream>>>((const bf16*)in, ld, CONV_ARGS, (float*)out, ld_out, n_rows, C, K, shift, act, residual);
+    else causal_conv_vec8_kernel<bf16><<<grid, block, lds, stream>>>((const bf16*)in, ld, CONV_ARGS, (bf16*)out, ld_out, n_rows, C, K, shift, act, residual);
+  } else if (out_f32 || dtype == GIBBS_F32)
     BY_DTYPE(dtype, "causal_conv",
              (causal_conv_silu_kernel<float, float><<<rows, 256, 0, stream>>>((const float*)in, ld, CONV_ARGS, (float*)out, ld_out, C, K, shift, act, residual)),
              (causal_conv_silu_kernel<bf16, float><<<rows, 256, 0, stream>>>((const bf16*)in, ld, CONV_ARGS, (float*)out, ld_out, C, K, shift, act, residual)));
