@@ -466,7 +466,8 @@ GIBBS_EXPORT int gibbs_causal_conv(const void* in, long ld, int dtype, const flo
                 "causal_conv: bad operands rows=%d requests=%d C=%d K=%d", n_rows, n_req, C, K);
   const dim3 rows(n_rows, ceil_div(C, 256)), reqs(n_req, ceil_div(C, 256));
 #define CONV_ARGS taps, bias, state, slot_stride, row_req, cu, slot
-  const bool vec8 = dtype == GIBBS_BF16 && C % 8 == 0 && ld % 8 == 0 && ((uintptr_t)in % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
+  // (steps of few rows are served faster by the kernel with a thread per channel: more, shorter workgroups; measured at 8 rows)
+  const bool vec8 = dtype == GIBBS_BF16 && n_rows >= 64 && C % 8 == 0 && ld % 8 == 0 && ((uintptr_t)in % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
                     ld_out % (out_f32 ? 4 : 8) == 0 && slot_stride % 4 == 0 && ((uintptr_t)state % 16) == 0 && ((uintptr_t)bias % 16) == 0 && K <= 16;
   if (vec8) {
     const dim3 grid(ceil_div(n_rows, CONV_ROWS), ceil_div(C, CONV_LANES * 8)), block(CONV_LANES, CONV_ROWS);
