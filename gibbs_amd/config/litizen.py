@@ -40,9 +40,10 @@ MIXER_TYPES = ("attention", "attention_2", "mamba2")
 class LitizenConfig(ArchConfig):
     architecture = "Litizen"
 
-    def __init__(self, cfg: Dict[str, Any], absent: Sequence[str] = ()):
+    def __init__(self, cfg: Dict[str, Any], absent: Sequence[str] = (), unread: Sequence[Tuple[str, Tuple[int, ...]]] = ()):
         self.cfg = cfg
         self.absent = frozenset(absent)     # optional tensors that the checkpoint does not hold
+        self.unread = tuple(unread)         # (name, shape) of checkpoint tensors of parts that a layer does not have
 
     def __eq__(self, other) -> bool:
         return isinstance(other, LitizenConfig) and self.cfg == other.cfg
@@ -66,7 +67,7 @@ class LitizenConfig(ArchConfig):
         layers = require(c, "layers")
         if not isinstance(layers, list) or not layers:
             raise ConfigError("config.json: layers must be a non-empty list")
-        optional = ["head"]
+        optional, unread = ["head"], []
         for i, layer in enumerate(layers):
             kind, m = layer.get("type"), layer.get("mixer")
             if kind not in MIXER_TYPES:
@@ -104,6 +105,8 @@ class LitizenConfig(ArchConfig):
                 optional += [p + "mix.g"] + ([p + "mix.q.norm", p + "mix.k.norm"] if kind == "attention" else [p + "mix.sink"])
             mlp = layer.get("mlp")
             if mlp is None:
+                if tensors is not None:      # (a layer without a feed-forward whose checkpoint holds that sublayer's norms all the same)
+                    unread += [(n, tuple(int(s) for s in tensors[n])) for n in (p + "norm2", p + "norm2b") if n in tensors]
                 continue
             if mlp.get("kind") == "dense":
                 int(require(mlp, "ff"))
@@ -123,7 +126,7 @@ class LitizenConfig(ArchConfig):
             absent += [n for n in optional if n.endswith(".canon1") and n not in absent]
         elif tensors is not None and any(n.endswith(".canon1") for n in absent) and not all(f"l{i}.canon1" in absent for i in range(len(layers))):
             raise ConfigError("the checkpoint holds an input convolution for some layers and not for others")
-        return cls(c, absent)
+        return cls(c, absent, unread)
 
     def to_dict(self) -> dict:
         return copy.deepcopy(self.cfg)
@@ -203,4 +206,5 @@ class LitizenConfig(ArchConfig):
         return ModelSpec(
             architecture=self.architecture, hidden=int(c["width"]), vocab=int(c["vocab"]), layers=tuple(layers), order=tuple(range(len(layers))),
             embedding="embed", final_norm=self.norm("final.norm"), head="head" if self._has("head") else None, max_position=MAX_POSITIONS,
-            embedding_scale=float((c.get("embedding") or {}).get("scale", 1.0)), logit_softcap=float(c.get("logit_softcap") or 0.0))
+            embedding_scale=float((c.get("embedding") or {}).get("scale", 1.0)), logit_softcap=float(c.get("logit_softcap") or 0.0),
+            unread_tensors=self.unread)

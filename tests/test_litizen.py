@@ -89,6 +89,10 @@ def test_what_the_checkpoint_holds_decides_the_optional_tensors():
     assert "mixer_input" not in [r for r, _ in spec.layers[0].parts]
     assert spec.layers[0].part("mixer").params.get("qk_norm") is None and spec.layers[2].part("mixer").params["sink"] is False
     assert spec.layers[2].part("mixer").params["gate"] is False and "correction" not in spec.layers[1].part("ffn").tensors
+    # a layer without a feed-forward whose checkpoint holds that sublayer's norms: declared, and read by nobody
+    more = dict(full, **{"l2.norm2": (100,), "l2.norm2b": (100,)})
+    spec = config_from_dict(LH.LITIZEN_A, tensors=more).model_spec()
+    assert {d.name for d in DecoderModel(spec).tensor_decls()} == set(more) and [r for r, _ in spec.layers[2].parts][-1] == "norm1b"
 
 
 @pytest.mark.parametrize("change, words", [

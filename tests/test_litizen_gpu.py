@@ -230,7 +230,7 @@ def _dev(a, dtype=torch.float32):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("case", [(100, 5, 1), (100, 1, 4), (96, 8, 3), (4096, 4, 4), (48, 48, 2)])
+@pytest.mark.parametrize("case", [(100, 5, 1), (100, 1, 4), (96, 8, 3), (4096, 4, 4), (48, 48, 2), (90, 5, 3), (9000, 2, 8)])
 def test_norm_in_groups_alone_added_and_both(dtype, case):
     """x += norm(delta) in `gd` parts and out = norm(x) in `gn` parts, each alone and in one pass; a part whose values are
     a thousand times the others' must not change its neighbours' scale; the tail's gather of rows."""
@@ -443,7 +443,7 @@ def test_keys_just_inside_and_just_outside_a_window_and_a_chunk(kernel, mask):
         assert hit == (far >= first_seen), f"head 2 and the key at {far} (the first key seen is {first_seen})"
 
 
-@pytest.mark.parametrize("sizes", [(3, 3, 7, 10), (4, 2, 48, 48), (2, 1, 128, 64), (8, 2, 16, 24)])
+@pytest.mark.parametrize("sizes", [(3, 3, 7, 10), (4, 2, 48, 48), (2, 1, 128, 64), (8, 2, 16, 24), (2, 1, 200, 8)])
 def test_state_written_long_ago_read_back_through_portions_and_a_reused_slot(sizes):
     """The state-space rule alone: one token's write (all other tokens' B are zero, decays of nearly one) is read back 400
     tokens later by a C that matches it, through portions of 1 to 150 tokens; the same walk in one step gives the same
