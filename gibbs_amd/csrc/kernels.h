@@ -112,7 +112,12 @@ int gibbs_causal_conv(const void* in, long ld, int dtype, const float* taps, con
                       const int* row_req, const int* cu, const int* slot, void* out, int out_f32, long ld_out, int n_rows, int n_req,
                       int C, int K, int act, int residual, int update_state, int single_rows, hipStream_t stream);
 int gibbs_ssd_prep(const float* xbc, long ld_x, const void* dt_raw, long ld_raw, int dtype, const float* dt_bias, const float* a_log,
-                   float* decay, float* xdt, int n_rows, int H, int V, hipStream_t stream);
+                   float* decay, float* log_decay, float* xdt, int n_rows, int H, int V, hipStream_t stream);
+// ---- ssd_chunked.hip: the same rule in chunks of 64 tokens, for one request's long stretch of rows
+long gibbs_ssd_chunked_workspace(int rows, int H, int D, int V);
+int gibbs_ssd_chunked(const float* q, const float* k, long ldqk, const float* v, long ldv, const float* log_decay, float* state,
+                      long slot_stride, const int* slot, float* out, float* workspace, int rows, int H, int G, int D, int V,
+                      hipStream_t stream);
 int gibbs_ssd_rule(const float* q, const float* k, long ldqk, const float* v, long ldv, const float* decay, float* state,
                    long slot_stride, const int* cu, const int* slot, float* out, int n_req, int H, int G, int D, int V,
                    hipStream_t stream);

@@ -522,21 +522,26 @@ int check_recurrence(const char* what, int n_req, int H, int G, int D, int V, lo
 template <typename T>
 __global__ void ssd_prep_kernel(const float* __restrict__ xbc, long ld_x, const T* __restrict__ dt_raw, long ld_raw,
                                 const float* __restrict__ dt_bias, const float* __restrict__ a_log, float* __restrict__ decay,
-                                float* __restrict__ xdt, int H, int V) {
+                                float* __restrict__ log_decay, float* __restrict__ xdt, int H, int V) {
   const int n = blockIdx.x, h = blockIdx.y;
   const float dt = softplus_f(to_float(dt_raw[(size_t)n * ld_raw + h]) + dt_bias[h]);
-  if (threadIdx.x == 0) decay[(size_t)n * H + h] = expf(-expf(a_log[h]) * dt);
+  if (threadIdx.x == 0) {
+    const float la = -expf(a_log[h]) * dt;
+    decay[(size_t)n * H + h] = expf(la);
+    if (log_decay) log_decay[(size_t)n * H + h] = la;
+  }
   for (int j = threadIdx.x; j < V; j += blockDim.x) xdt[(size_t)n * H * V + (size_t)h * V + j] = dt * xbc[(size_t)n * ld_x + (size_t)h * V + j];
 }
+// (log_decay [N, H], optional: the decay's logarithm, -exp(a_log) dt, for the rule in chunks)
 GIBBS_EXPORT int gibbs_ssd_prep(const float* xbc, long ld_x, const void* dt_raw, long ld_raw, int dtype, const float* dt_bias,
-                                const float* a_log, float* decay, float* xdt, int n_rows, int H, int V, hipStream_t stream) {
+                                const float* a_log, float* decay, float* log_decay, float* xdt, int n_rows, int H, int V, hipStream_t stream) {
   GIBBS_REQUIRE(xbc && dt_raw && dt_bias && a_log && decay && xdt && n_rows > 0 && H > 0 && V > 0 && ld_x >= (long)H * V && ld_raw >= H,
                 "ssd_prep: bad operands rows=%d heads=%d V=%d", n_rows, H, V);
   GIBBS_REQUIRE(H <= 65535, "ssd_prep: too many heads (%d)", H);
   const dim3 grid(n_rows, H);
   BY_DTYPE(dtype, "ssd_prep",
-           (ssd_prep_kernel<float><<<grid, WAVE, 0, stream>>>(xbc, ld_x, (const float*)dt_raw, ld_raw, dt_bias, a_log, decay, xdt, H, V)),
-           (ssd_prep_kernel<bf16><<<grid, WAVE, 0, stream>>>(xbc, ld_x, (const bf16*)dt_raw, ld_raw, dt_bias, a_log, decay, xdt, H, V)));
+           (ssd_prep_kernel<float><<<grid, WAVE, 0, stream>>>(xbc, ld_x, (const float*)dt_raw, ld_raw, dt_bias, a_log, decay, log_decay, xdt, H, V)),
+           (ssd_prep_kernel<bf16><<<grid, WAVE, 0, stream>>>(xbc, ld_x, (const bf16*)dt_raw, ld_raw, dt_bias, a_log, decay, log_decay, xdt, H, V)));
   GIBBS_LAUNCH_STATUS("ssd_prep");
 }
 

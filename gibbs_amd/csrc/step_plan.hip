@@ -47,6 +47,7 @@ constexpr int FUSED_ROWS = 64;            // rows that the few-row products (and
 constexpr int SKINNY_ROWS = 64;           // rows up to which a plain product takes the weight-streaming kernel
 constexpr int SKINNY_ROWS_F32_OUT = 48;   // the same for float32 output (the head: it streams faster than the tiled product)
 constexpr int ACT_CLAMPED = 4;            // the gated feed-forward's clamped activation (activation.h: ACT_CLAMPED_SWISH)
+constexpr int SSD_CHUNKED_ROWS = 256;     // rows of one request from which the state-space rule runs in chunks
 constexpr int MATRIX_SLICE_PAGES = 510;   // page ids of a key slice that the decode attention's matrix-core walk keeps in LDS
 
 // Ranges of k that the few-row product is cut into so that at least `want_blocks` workgroups run (a
@@ -857,12 +858,24 @@ struct SsdBody : Body {
     float* xbc = (float*)e.take((long)N * C * 4);
     RUN(e, gibbs_causal_conv(raw + (long)inner * e.esize, in.O, e.p.dtype, taps, conv_bias, conv_state, slot_stride, a.row_req, a.cu, a.slot, xbc, 1, C,
                              N, a.n_req, C, K, 1, 0, 1, a.max_q == 1, a.stream));
+    // one request's long portion takes the rule in chunks (matrix products over 64 tokens at a time; it agrees with the walk
+    // to rounding); everything else walks token by token
+    const long chunk_floats = (a.n_req == 1 && N >= SSD_CHUNKED_ROWS && C % 4 == 0 && (G * D) % 4 == 0) ? gibbs_ssd_chunked_workspace(N, H, D, V) : 0;
     float* decay = (float*)e.take((long)N * H * 4);
+    float* log_decay = chunk_floats ? (float*)e.take((long)N * H * 4) : nullptr;
     float* xdt = (float*)e.take((long)N * inner * 4);
-    RUN(e, gibbs_ssd_prep(xbc, C, raw + (long)(inner + C) * e.esize, in.O, e.p.dtype, dt_bias, a_log, decay, xdt, N, H, V, a.stream));
+    RUN(e, gibbs_ssd_prep(xbc, C, raw + (long)(inner + C) * e.esize, in.O, e.p.dtype, dt_bias, a_log, decay, log_decay, xdt, N, H, V, a.stream));
     float* o = (float*)e.take((long)N * inner * 4);
-    RUN(e, gibbs_ssd_rule(xbc + inner + (long)G * D, xbc + inner, C, xdt, inner, decay, rule_state, slot_stride, a.cu, a.slot, o, a.n_req, H, G, D, V,
-                          a.stream));
+    if (chunk_floats) {
+      float* work = (float*)e.take(chunk_floats * 4);
+      RUN(e, gibbs_ssd_chunked(xbc + inner + (long)G * D, xbc + inner, C, xdt, inner, log_decay, rule_state, slot_stride, a.slot, o, work, N, H, G, D, V,
+                               a.stream));
+      e.give(work);
+      e.give(log_decay);
+    } else {
+      RUN(e, gibbs_ssd_rule(xbc + inner + (long)G * D, xbc + inner, C, xdt, inner, decay, rule_state, slot_stride, a.cu, a.slot, o, a.n_req, H, G, D, V,
+                            a.stream));
+    }
     e.give(decay);
     e.give(xdt);
     void* y = e.take((long)N * inner * e.esize);

@@ -86,7 +86,9 @@ _SIGNATURES = {
                                c_int, c_void_p],
     "gibbs_causal_conv": [c_void_p, c_long, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_long,
                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
-    "gibbs_ssd_prep": [c_void_p, c_long, c_void_p, c_long, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "gibbs_ssd_prep": [c_void_p, c_long, c_void_p, c_long, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "gibbs_ssd_chunked": [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                          c_int, c_int, c_void_p],
     "gibbs_ssd_rule": [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
                        c_int, c_int, c_int, c_void_p],
     "gibbs_moe_route_mode": [c_void_p, c_long, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
@@ -158,6 +160,7 @@ _VALUE_SIGNATURES = {
     "gibbs_rule_fused_rows": ([], c_int),
     "gibbs_linear_splits": ([c_int, c_int, c_int, c_int, c_long, c_void_p, c_void_p, c_int, c_int, c_int], c_int),
     "gibbs_skinny_residual_workspace": ([c_int, c_int, c_int], c_long),
+    "gibbs_ssd_chunked_workspace": ([c_int, c_int, c_int, c_int], c_long),
 }
 
 

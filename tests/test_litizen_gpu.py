@@ -549,6 +549,66 @@ def test_scores_over_all_experts_corrections_identity_experts_and_the_sum(case):
     assert np.abs(out.float().cpu().numpy() - want).max() <= tol * np.abs(want).max()
 
 
+@pytest.mark.parametrize("sizes", [(3, 3, 8, 12, 300), (4, 2, 48, 48, 257), (2, 1, 128, 64, 640), (2, 2, 20, 100, 450), (1, 1, 4, 4, 64)])
+def test_the_rule_in_chunks_against_the_walk(sizes):
+    """One request's long stretch of rows through the rule in chunks of 64 tokens (sizes that are no multiples of 64,
+    more columns than a workgroup takes, a last chunk that is not full), from a state that an earlier call left: the plain
+    recurrence's read-outs and state, and the token-by-token kernel's, to rounding; decays from nearly one down to 1e-4 a token."""
+    from gibbs_amd.ops.lib import call, library, ptr, stream
+    H, G, D, V, T = sizes
+    rng = np.random.default_rng(6)
+    first = 37
+    n = first + T
+    B, C, x = rng.normal(size=(n, G, D)), rng.normal(size=(n, G, D)), rng.normal(size=(n, H, V))
+    dt = rng.uniform(0.05, 1.5, size=(n, H))
+    a_log = np.linspace(-6.0, 1.8, H)
+    log_decay = -np.exp(a_log)[None, :] * dt
+    want = Z.ssd_scan(x, B, C, dt, a_log, np.zeros(H), G)
+    bc = _dev(np.concatenate([B.reshape(n, -1), C.reshape(n, -1)], axis=1))
+    xdt = _dev((x * dt[:, :, None]).reshape(n, -1))
+    decay, logd = _dev(np.exp(log_decay)), _dev(log_decay)
+    slot = _dev([1], torch.int32)
+
+    def walk(state, a, b, out):
+        call("gibbs_ssd_rule", bc[a:b].data_ptr() + G * D * 4, bc[a:b].data_ptr(), 2 * G * D, xdt[a:b].data_ptr(), H * V, decay[a:b].data_ptr(), ptr(state),
+             state.stride(0), ptr(_dev([0, b - a], torch.int32)), ptr(slot), out[a:b].data_ptr(), 1, H, G, D, V, stream())
+
+    state_w = torch.zeros((3, H * D * V + 5), dtype=torch.float32, device="cuda")
+    out_w = torch.zeros((n, H * V), dtype=torch.float32, device="cuda")
+    walk(state_w, 0, first, out_w)
+    state_c = state_w.clone()
+    out_c = out_w.clone()
+    walk(state_w, first, n, out_w)
+    floats = library().gibbs_ssd_chunked_workspace(T, H, D, V)
+    assert floats > 0
+    work = torch.full((floats,), float("nan"), dtype=torch.float32, device="cuda")
+    call("gibbs_ssd_chunked", bc[first:].data_ptr() + G * D * 4, bc[first:].data_ptr(), 2 * G * D, xdt[first:].data_ptr(), H * V, logd[first:].data_ptr(),
+         ptr(state_c), state_c.stride(0), ptr(slot), out_c[first:].data_ptr(), ptr(work), T, H, G, D, V, stream())
+    scale = np.abs(want).max()
+    assert np.abs(out_w.cpu().numpy().reshape(n, H, V) - want).max() <= 3e-5 * scale
+    assert np.abs(out_c.cpu().numpy().reshape(n, H, V) - want).max() <= 3e-5 * scale
+    assert torch.isfinite(state_c).all() and (state_c[1] - state_w[1]).abs().max() <= 3e-5 * state_w[1].abs().max()
+    assert not state_c[0].any() and not state_c[2].any() and not state_c[1, H * D * V:].any()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_long_prompt_whole_in_portions_and_decoded(dirs, dtype, tmp_path):
+    """A prompt long enough for the state-space rule's chunks (600 tokens in one step), the same prompt in portions that are
+    too short for them, and its last tokens one by one: all against the plain logits."""
+    cfg = {"architecture": "Litizen", "vocab": 150, "width": 64, "norm": {"eps": 1e-5, "groups": 2}, "canon": {"taps": 3},
+           "layers": [LH.with_mlp(LH.state_space(4, 16, 24, 2, 4, 2), LH.dense(96)), LH.with_mlp(LH.chunk_attention(4, 2, 16, 16, 0.25, 1e4, dims=8, size=150), None),
+                      LH.with_mlp(LH.state_space(3, 8, 128, 1, 2, 1), LH.dense(64))]}
+    d = LH.make_model_dir(str(tmp_path), cfg, "long", seed=12)
+    ids = LH.tokens(8, 600, 150)
+    want = [0, 63, 64, 255, 256, 300, 511, 512, 598, 599]
+    whole = run_steps(make_engine(d, dtype), [([("r", ids, want)], ["r"])])
+    check(d, {"r": ids}, whole, dtype, f"long prompt whole {dtype}")
+    cuts = portions(560, [200, 90, 255, 15]) + [(560 + i, 561 + i) for i in range(40)]
+    cut = run_steps(make_engine(d, dtype), [([("r", ids[a:b], [p - a for p in want if a <= p < b])], []) for a, b in cuts])
+    check(d, {"r": ids}, cut, dtype, f"long prompt in portions {dtype}")
+    assert sorted(cut) == sorted(whole)
+
+
 # ----------------------------------------------------------------------------------------------- entry points
 def plain_greedy(model_dir, prompt, n):
     ids = list(prompt)
