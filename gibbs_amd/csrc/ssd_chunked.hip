@@ -15,7 +15,8 @@ constexpr int L = 64, VB = 64, DMAX = 128, NT = 256;
 constexpr int RT = L * 16 / NT;        // rows of a thread's RT x 4 tile of a 64 x 64 result (16 threads across the columns)
 constexpr int ROWG = NT / 16;          // row groups of the tiles
 constexpr int VEC_LOADS = L * DMAX / 4 / NT;   // 16-byte vectors a thread brings in for a 64 x 128 operand
-constexpr int LDQ = DMAX + 4, LDV = VB + 4, LDG = L + 4;
+constexpr int DH = 64;                 // channels of Q and K that the local kernel holds in LDS at a time
+constexpr int LDQ = DMAX + 4, LDH = DH + 4, LDV = VB + 4, LDG = L + 4;
 
 struct ChunkArgs {
   const float* q; const float* k; long ldqk;      // [rows, G * D]: C and B of the rows
@@ -59,104 +60,102 @@ __device__ __forceinline__ void load_rows(const float* src, long ld, int c0, int
 }
 
 __global__ __launch_bounds__(NT) void ssd_chunk_local_kernel(ChunkArgs a) {
+  // Q and K come through LDS in halves of 64 channels (70 KB in all: two workgroups a compute unit, so that one's waits
+  // for LDS are the other's arithmetic); the scores' tile stays in registers across the halves.
   extern __shared__ float lds[];
-  float* sQ = lds;                    // [L][LDQ]
-  float* sK = sQ + L * LDQ;           // [L][LDQ]
-  float* sV = sK + L * LDQ;           // [L][LDV]
+  float* sQ = lds;                    // [L][LDH]: 64 channels of Q
+  float* sK = sQ + L * LDH;           // [L][LDH]
+  float* sV = sK + L * LDH;           // [L][LDV]
   float* sG = sV + L * LDV;           // [L][LDG]
   float* cum = sG + L * LDG;          // [L]
   float* sW = cum + L;                // [L]: exp(c_L - c_s)
   const int chunk = blockIdx.x, h = blockIdx.y, j0 = blockIdx.z * VB;
-  const int t0 = chunk * L, g = h / (a.H / a.G), D = a.D, Dp = (D + 3) / 4 * 4;
+  const int t0 = chunk * L, g = h / (a.H / a.G), D = a.D;
   const int vw = min(VB, a.V - j0);
+  const int ty = threadIdx.x / 16, tx = threadIdx.x % 16;      // an RT x 4 tile of a 64 x 64 result
   chunk_sums(a, t0, h, cum);
-  load_rows(a.q, a.ldqk, g * D, D, Dp, t0, a.rows, sQ, LDQ);
-  load_rows(a.k, a.ldqk, g * D, D, Dp, t0, a.rows, sK, LDQ);
   load_rows(a.v, a.ldv, h * a.V + j0, vw, VB, t0, a.rows, sV, LDV);
   __syncthreads();
   if (blockIdx.z == 0 && threadIdx.x == 0) a.total_log[(size_t)chunk * a.H + h] = cum[L - 1];
   if (threadIdx.x < L) sW[threadIdx.x] = expf(cum[L - 1] - cum[threadIdx.x]);      // (read behind the next barrier)
-  const int ty = threadIdx.x / 16, tx = threadIdx.x % 16;      // an RT x 4 tile of a 64 x 64 result
-  // G[t][s] = exp(c_t - c_s) (q_t . k_s) for s <= t
-  {
-    float acc[RT][4] = {};
-    for (int d = 0; d < Dp; d += 4) {
+  float* u = a.u + ((size_t)chunk * a.H + h) * D * a.V;
+  float gacc[RT][4] = {};
+  for (int d0 = 0; d0 < D; d0 += DH) {
+    const int dw = min(DH, D - d0);
+    __syncthreads();      // (everyone is done with the half before)
+    load_rows(a.q, a.ldqk, g * D + d0, dw, DH, t0, a.rows, sQ, LDH);
+    load_rows(a.k, a.ldqk, g * D + d0, dw, DH, t0, a.rows, sK, LDH);
+    __syncthreads();
+    // G[t][s] += q_t . k_s over this half's channels
+    for (int d = 0; d < DH; d += 4) {
       float4 qa[RT], kb[4];
 #pragma unroll
-      for (int i = 0; i < RT; ++i) qa[i] = *(const float4*)&sQ[(RT * ty + i) * LDQ + d];
+      for (int i = 0; i < RT; ++i) qa[i] = *(const float4*)&sQ[(RT * ty + i) * LDH + d];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) kb[i] = *(const float4*)&sK[(4 * tx + i) * LDQ + d];
+      for (int i = 0; i < 4; ++i) kb[i] = *(const float4*)&sK[(4 * tx + i) * LDH + d];
 #pragma unroll
       for (int i = 0; i < RT; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          acc[i][j] = fmaf(qa[i].x, kb[j].x, acc[i][j]); acc[i][j] = fmaf(qa[i].y, kb[j].y, acc[i][j]);
-          acc[i][j] = fmaf(qa[i].z, kb[j].z, acc[i][j]); acc[i][j] = fmaf(qa[i].w, kb[j].w, acc[i][j]);
+          gacc[i][j] = fmaf(qa[i].x, kb[j].x, gacc[i][j]); gacc[i][j] = fmaf(qa[i].y, kb[j].y, gacc[i][j]);
+          gacc[i][j] = fmaf(qa[i].z, kb[j].z, gacc[i][j]); gacc[i][j] = fmaf(qa[i].w, kb[j].w, gacc[i][j]);
         }
     }
-#pragma unroll
-    for (int i = 0; i < RT; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int t = RT * ty + i, s = 4 * tx + j;
-        sG[t * LDG + s] = s <= t ? acc[i][j] * expf(cum[t] - cum[s]) : 0.f;
-      }
-  }
-  __syncthreads();
-  // Y[t][j] = sum_s G[t][s] V[s][j]
-  {
-    float acc[RT][4] = {};
-    for (int s = 0; s < L; s += 4) {
-      float4 ga[RT], vb[4];
-#pragma unroll
-      for (int i = 0; i < RT; ++i) ga[i] = *(const float4*)&sG[(RT * ty + i) * LDG + s];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) vb[i] = *(const float4*)&sV[(s + i) * LDV + 4 * tx];
-#pragma unroll
-      for (int i = 0; i < RT; ++i) {
-        const float gs[4] = {ga[i].x, ga[i].y, ga[i].z, ga[i].w};
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-          acc[i][0] = fmaf(gs[kk], vb[kk].x, acc[i][0]); acc[i][1] = fmaf(gs[kk], vb[kk].y, acc[i][1]);
-          acc[i][2] = fmaf(gs[kk], vb[kk].z, acc[i][2]); acc[i][3] = fmaf(gs[kk], vb[kk].w, acc[i][3]);
-        }
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < RT; ++i) {
-      const int t = t0 + RT * ty + i;
-      if (t >= a.rows) continue;
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (4 * tx + j < vw) a.out[(size_t)t * a.H * a.V + (size_t)h * a.V + j0 + 4 * tx + j] = acc[i][j];
-    }
-  }
-  // U[i][j] = sum_s exp(c_L - c_s) K[s][i] V[s][j]: 4 columns of V by DMAX / ROWG rows of the state a thread (i = ty + ROWG m)
-  {
-    float acc[DMAX / ROWG][4] = {};
+    // U[i][j] = sum_s exp(c_L - c_s) K[s][i] V[s][j] for this half's rows i = d0 + ty + ROWG m: 4 columns of V a thread
+    float acc[DH / ROWG][4] = {};
     for (int s = 0; s < L; ++s) {
       const float w = sW[s];
       const float4 vb = *(const float4*)&sV[s * LDV + 4 * tx];
       const float4 wv = make_float4(w * vb.x, w * vb.y, w * vb.z, w * vb.w);
 #pragma unroll
-      for (int m = 0; m < DMAX / ROWG; ++m) {
-        const int i = ty + ROWG * m;
-        if (i < D) {
-          const float kv = sK[s * LDQ + i];
-          acc[m][0] = fmaf(kv, wv.x, acc[m][0]); acc[m][1] = fmaf(kv, wv.y, acc[m][1]);
-          acc[m][2] = fmaf(kv, wv.z, acc[m][2]); acc[m][3] = fmaf(kv, wv.w, acc[m][3]);
-        }
+      for (int m = 0; m < DH / ROWG; ++m) {
+        const float kv = sK[s * LDH + ty + ROWG * m];
+        acc[m][0] = fmaf(kv, wv.x, acc[m][0]); acc[m][1] = fmaf(kv, wv.y, acc[m][1]);
+        acc[m][2] = fmaf(kv, wv.z, acc[m][2]); acc[m][3] = fmaf(kv, wv.w, acc[m][3]);
       }
     }
-    float* u = a.u + ((size_t)chunk * a.H + h) * D * a.V;
 #pragma unroll
-    for (int m = 0; m < DMAX / ROWG; ++m) {
-      const int i = ty + ROWG * m;
+    for (int m = 0; m < DH / ROWG; ++m) {
+      const int i = d0 + ty + ROWG * m;
       if (i >= D) continue;
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         if (4 * tx + j < vw) u[(size_t)i * a.V + j0 + 4 * tx + j] = acc[m][j];
     }
+  }
+#pragma unroll
+  for (int i = 0; i < RT; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int t = RT * ty + i, s = 4 * tx + j;
+      sG[t * LDG + s] = s <= t ? gacc[i][j] * expf(cum[t] - cum[s]) : 0.f;
+    }
+  __syncthreads();
+  // Y[t][j] = sum_s G[t][s] V[s][j]
+  float acc[RT][4] = {};
+  for (int s = 0; s < L; s += 4) {
+    float4 ga[RT], vb[4];
+#pragma unroll
+    for (int i = 0; i < RT; ++i) ga[i] = *(const float4*)&sG[(RT * ty + i) * LDG + s];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) vb[i] = *(const float4*)&sV[(s + i) * LDV + 4 * tx];
+#pragma unroll
+    for (int i = 0; i < RT; ++i) {
+      const float gs[4] = {ga[i].x, ga[i].y, ga[i].z, ga[i].w};
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        acc[i][0] = fmaf(gs[kk], vb[kk].x, acc[i][0]); acc[i][1] = fmaf(gs[kk], vb[kk].y, acc[i][1]);
+        acc[i][2] = fmaf(gs[kk], vb[kk].z, acc[i][2]); acc[i][3] = fmaf(gs[kk], vb[kk].w, acc[i][3]);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < RT; ++i) {
+    const int t = t0 + RT * ty + i;
+    if (t >= a.rows) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (4 * tx + j < vw) a.out[(size_t)t * a.H * a.V + (size_t)h * a.V + j0 + 4 * tx + j] = acc[i][j];
   }
 }
 
@@ -258,7 +257,7 @@ GIBBS_EXPORT int gibbs_ssd_chunked(const float* q, const float* k, long ldqk, co
   GIBBS_REQUIRE(H <= 65535 && ceil_div(V, VB) <= 65535, "ssd_chunked: too many heads or columns");
   ChunkArgs a{q, k, ldqk, v, ldv, log_decay, workspace, workspace + (size_t)chunks * H * D * V, state, slot_stride, slot, out, rows, H, G, D, V};
   const dim3 grid(chunks, H, ceil_div(V, VB));
-  const size_t lds_local = (size_t)(2 * L * LDQ + L * LDV + L * LDG + 2 * L) * sizeof(float);
+  const size_t lds_local = (size_t)(2 * L * LDH + L * LDV + L * LDG + 2 * L) * sizeof(float);
   const size_t lds_carry = (size_t)(L * LDQ + DMAX * LDV + L) * sizeof(float);
   static bool raised = false;
   if (!raised) {
