@@ -115,6 +115,8 @@ int gibbs_ssd_prep(const float* xbc, long ld_x, const void* dt_raw, long ld_raw,
                    float* decay, float* log_decay, float* xdt, int n_rows, int H, int V, hipStream_t stream);
 // ---- ssd_chunked.hip: the same rule in chunks of 64 tokens, for one request's long stretch of rows
 long gibbs_ssd_chunked_workspace(int rows, int H, int D, int V);
+int gibbs_ssd_step(const float* q, const float* k, long ldqk, const float* v, long ldv, const float* decay, float* state, long slot_stride,
+                   const int* slot, float* out, int n_req, int H, int G, int D, int V, hipStream_t stream);
 int gibbs_ssd_chunked(const float* q, const float* k, long ldqk, const float* v, long ldv, const float* log_decay, float* state,
                       long slot_stride, const int* slot, float* out, float* workspace, int rows, int H, int G, int D, int V,
                       hipStream_t stream);

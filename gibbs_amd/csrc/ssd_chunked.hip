@@ -3,6 +3,7 @@
 // regrouped so that every product is a small matrix product and only a sum over chunks runs in order.  With chunks of
 // L = 64 tokens, c_t = sum of log a over the chunk's tokens up to t, and S_0 the state in front of the chunk:
 //   y_t = exp(c_t) S_0' q_t + sum_(s <= t) exp(c_t - c_s) (k_s . q_t) v_s         S_L = exp(c_L) S_0 + sum_s exp(c_L - c_s) k_s v_s'
+// (A step of one token per request has a kernel of its own at the end of this file.)
 // Three kernels: (1) per (chunk, head, 64 columns of V): G = mask .* (Q K'), Y = G V, and the chunk's own contribution
 // U = K' diag(exp(c_L - c_s)) V; (2) per element of the state, over the chunks in order: what stood in front of each
 // chunk (written where U was) and the state behind the last; (3) per (chunk, head, columns): Y += diag(exp(c_t)) Q S_0.
@@ -233,6 +234,41 @@ __global__ __launch_bounds__(NT) void ssd_chunk_carry_kernel(ChunkArgs a) {
       }
   }
 }
+// One token per request (a step of decoded tokens): the state is streamed once, in whole rows.  A workgroup takes 64 columns
+// of one head's state; thread (lane, part) owns column j and the rows i = part, part + STEP_PARTS, ...: S_ij = a S_ij + k_i v_j
+// (the walk's own arithmetic, so the state is the walk's to the bit), y_j = sum_i S_ij q_i by parts that are added in order.
+constexpr int STEP_PARTS = 4;
+__global__ __launch_bounds__(64 * STEP_PARTS) void ssd_step_kernel(const float* __restrict__ q, const float* __restrict__ k, long ldqk,
+                                                                   const float* __restrict__ v, long ldv, const float* __restrict__ decay,
+                                                                   float* __restrict__ state, long slot_stride, const int* __restrict__ slot,
+                                                                   float* __restrict__ out, int H, int G, int D, int V) {
+  __shared__ float sq[256], sk[256], sy[STEP_PARTS][64];
+  const int n = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, part = threadIdx.y;
+  const int j = blockIdx.z * 64 + lane, g = h / (H / G);
+  for (int i = part * 64 + lane; i < D; i += 64 * STEP_PARTS) {
+    sq[i] = q[(size_t)n * ldqk + (size_t)g * D + i];
+    sk[i] = k[(size_t)n * ldqk + (size_t)g * D + i];
+  }
+  __syncthreads();
+  float y = 0.f;
+  if (j < V) {
+    const float a = decay[(size_t)n * H + h], vj = v[(size_t)n * ldv + (size_t)h * V + j];
+    float* st = state + (size_t)slot[n] * slot_stride + (size_t)h * D * V + j;
+    for (int i = part; i < D; i += STEP_PARTS) {
+      const float s = fmaf(a, st[(size_t)i * V], sk[i] * vj);
+      st[(size_t)i * V] = s;
+      y = fmaf(s, sq[i], y);
+    }
+  }
+  sy[part][lane] = y;
+  __syncthreads();
+  if (part == 0 && j < V) {
+    float total = sy[0][lane];
+#pragma unroll
+    for (int p = 1; p < STEP_PARTS; ++p) total += sy[p][lane];
+    out[(size_t)n * H * V + (size_t)h * V + j] = total;
+  }
+}
 }  // namespace
 
 // Floats of workspace that `rows` rows of one request need (0: the chunked form does not take these sizes).
@@ -271,4 +307,16 @@ GIBBS_EXPORT int gibbs_ssd_chunked(const float* q, const float* k, long ldqk, co
   ssd_chunk_scan_kernel<<<ceil_div(total, 256), 256, 0, stream>>>(a, chunks);
   ssd_chunk_carry_kernel<<<grid, NT, lds_carry, stream>>>(a);
   GIBBS_LAUNCH_STATUS("ssd_chunked");
+}
+
+// The rule for a step in which every request brings one row (row n is request n): q, k [n_req, >= G D], v [n_req, >= H V], decay
+// [n_req, H], the requests' states at state + slot[n] * slot_stride, out [n_req, H V].  All float32; D up to 256.
+GIBBS_EXPORT int gibbs_ssd_step(const float* q, const float* k, long ldqk, const float* v, long ldv, const float* decay, float* state,
+                                long slot_stride, const int* slot, float* out, int n_req, int H, int G, int D, int V, hipStream_t stream) {
+  GIBBS_REQUIRE(q && k && v && decay && state && slot && out && n_req > 0, "ssd_step: null operand or no rows");
+  GIBBS_REQUIRE(H > 0 && G > 0 && H % G == 0 && D > 0 && D <= 256 && V > 0 && ldqk >= (long)G * D && ldv >= (long)H * V && slot_stride >= (long)H * D * V,
+                "ssd_step: bad sizes heads=%d groups=%d D=%d (up to 256) V=%d", H, G, D, V);
+  GIBBS_REQUIRE(H <= 65535 && ceil_div(V, 64) <= 65535, "ssd_step: too many heads or columns");
+  ssd_step_kernel<<<dim3(n_req, H, ceil_div(V, 64)), dim3(64, STEP_PARTS), 0, stream>>>(q, k, ldqk, v, ldv, decay, state, slot_stride, slot, out, H, G, D, V);
+  GIBBS_LAUNCH_STATUS("ssd_step");
 }

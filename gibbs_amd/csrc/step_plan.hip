@@ -872,6 +872,9 @@ struct SsdBody : Body {
                                a.stream));
       e.give(work);
       e.give(log_decay);
+    } else if (a.max_q == 1 && a.n_rows == a.n_req) {
+      // one token per request: the kernel that streams the state in whole rows (the walk's arithmetic for the state itself)
+      RUN(e, gibbs_ssd_step(xbc + inner + (long)G * D, xbc + inner, C, xdt, inner, decay, rule_state, slot_stride, a.slot, o, a.n_req, H, G, D, V, a.stream));
     } else {
       RUN(e, gibbs_ssd_rule(xbc + inner + (long)G * D, xbc + inner, C, xdt, inner, decay, rule_state, slot_stride, a.cu, a.slot, o, a.n_req, H, G, D, V,
                             a.stream));

@@ -87,6 +87,8 @@ _SIGNATURES = {
     "gibbs_causal_conv": [c_void_p, c_long, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_long,
                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gibbs_ssd_prep": [c_void_p, c_long, c_void_p, c_long, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "gibbs_ssd_step": [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                       c_void_p],
     "gibbs_ssd_chunked": [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                           c_int, c_int, c_void_p],
     "gibbs_ssd_rule": [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,

@@ -549,6 +549,33 @@ def test_scores_over_all_experts_corrections_identity_experts_and_the_sum(case):
     assert np.abs(out.float().cpu().numpy() - want).max() <= tol * np.abs(want).max()
 
 
+@pytest.mark.parametrize("sizes", [(3, 3, 7, 10), (4, 2, 40, 56), (2, 1, 200, 72), (8, 2, 128, 64)])
+def test_one_token_per_request_against_the_walk(sizes):
+    """Three requests that bring one token each, for 20 steps, through the kernel for such steps and through the walk: the
+    states are equal to the bit (the same arithmetic per element), the read-outs to rounding; slots are scattered."""
+    from gibbs_amd.ops.lib import call, ptr, stream
+    H, G, D, V = sizes
+    rng = np.random.default_rng(8)
+    R, steps = 3, 20
+    slots = _dev([2, 0, 3], torch.int32)
+    cu = _dev([0, 1, 2, 3], torch.int32)
+    state_a = _dev(rng.normal(size=(5, H * D * V + 3)))
+    state_b = state_a.clone()
+    for _ in range(steps):
+        bc = _dev(rng.normal(size=(R, 2 * G * D)))
+        xdt = _dev(rng.normal(size=(R, H * V)))
+        decay = _dev(rng.uniform(0.2, 1.0, size=(R, H)))
+        out_a = torch.empty((R, H * V), dtype=torch.float32, device="cuda")
+        out_b = torch.empty_like(out_a)
+        call("gibbs_ssd_rule", bc.data_ptr() + G * D * 4, ptr(bc), 2 * G * D, ptr(xdt), H * V, ptr(decay), ptr(state_a), state_a.stride(0), ptr(cu), ptr(slots),
+             ptr(out_a), R, H, G, D, V, stream())
+        call("gibbs_ssd_step", bc.data_ptr() + G * D * 4, ptr(bc), 2 * G * D, ptr(xdt), H * V, ptr(decay), ptr(state_b), state_b.stride(0), ptr(slots),
+             ptr(out_b), R, H, G, D, V, stream())
+        assert torch.equal(state_a, state_b)
+        assert (out_a - out_b).abs().max() <= 2e-5 * out_a.abs().max()
+    assert torch.equal(state_a[1], state_b[1]) and torch.equal(state_a[4], state_b[4])      # slots of no request are untouched
+
+
 @pytest.mark.parametrize("sizes", [(3, 3, 8, 12, 300), (4, 2, 40, 56, 257), (2, 1, 128, 64, 640), (2, 2, 20, 100, 450), (1, 1, 4, 4, 64)])
 def test_the_rule_in_chunks_against_the_walk(sizes):
     """One request's long stretch of rows through the rule in chunks of 64 tokens (sizes that are no multiples of 64,
