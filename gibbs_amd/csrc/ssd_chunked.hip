@@ -254,10 +254,23 @@ __global__ __launch_bounds__(64 * STEP_PARTS) void ssd_step_kernel(const float* 
   if (j < V) {
     const float a = decay[(size_t)n * H + h], vj = v[(size_t)n * ldv + (size_t)h * V + j];
     float* st = state + (size_t)slot[n] * slot_stride + (size_t)h * D * V + j;
-    for (int i = part; i < D; i += STEP_PARTS) {
-      const float s = fmaf(a, st[(size_t)i * V], sk[i] * vj);
-      st[(size_t)i * V] = s;
-      y = fmaf(s, sq[i], y);
+    // (eight rows at a time: their loads are all asked for before the first store, which the compiler must take to alias them)
+    for (int i0 = part; i0 < D; i0 += 8 * STEP_PARTS) {
+      float s[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = i0 + u * STEP_PARTS;
+        s[u] = i < D ? st[(size_t)i * V] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = i0 + u * STEP_PARTS;
+        if (i < D) {
+          s[u] = fmaf(a, s[u], sk[i] * vj);
+          st[(size_t)i * V] = s[u];
+          y = fmaf(s[u], sq[i], y);
+        }
+      }
     }
   }
   sy[part][lane] = y;
